@@ -119,6 +119,16 @@ int32_t sz_exl3_codebook(uint64_t out_f32_65536, uint64_t stream);
 uint64_t sz_matvec_cols_scratch(int32_t ggml_type, uint64_t cols, uint64_t rows, uint32_t m);
 int32_t sz_matvec_cols(int32_t ggml_type, uint64_t w, uint64_t cols, uint64_t rows, uint64_t x, uint32_t xs, uint64_t y, uint32_t ys,
                        uint32_t m, uint64_t scratch, uint64_t scratch_bytes, uint64_t stream);
+/* sz_matvec_cols without a workspace argument and without any allocation.  No counterpart in the reference: it is for
+ * callers that cannot allocate device memory (code under HIP graph capture, serving loops, harnesses that forbid
+ * hipMalloc).  The workspace is a device array of SZ_STATIC_WORKSPACE_BYTES inside the library, one copy on every GPU the
+ * library runs on, held until the process ends; a product whose sz_matvec_cols_scratch() is larger is refused with an
+ * error before anything is launched (GGUF and unquantized types need none; an EXL3 expert projection needs tens of KB).
+ * Results are those of sz_matvec_cols, bit for bit.  All calls on one GPU share the array: calls that overlap in time on
+ * one GPU (two streams) race on it; calls on one stream are ordered and need nothing cleared between them. */
+#define SZ_STATIC_WORKSPACE_BYTES (4u << 20)
+int32_t sz_matvec_cols_static(int32_t ggml_type, uint64_t w, uint64_t cols, uint64_t rows, uint64_t x, uint32_t xs, uint64_t y, uint32_t ys,
+                              uint32_t m, uint64_t stream);
 
 /* ---- B2: the session's verify-path operations (crates/shadowzero-cuda/src/session.rs:6076, 8222-8285, 8871, 7034-7052) */
 typedef struct {

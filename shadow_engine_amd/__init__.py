@@ -136,6 +136,7 @@ _SIGNATURES = {
     "sz_exl3_codebook": (_i32, [_u64, _u64]),
     "sz_matvec_cols_scratch": (_u64, [_i32, _u64, _u64, _u32]),
     "sz_matvec_cols": (_i32, [_i32, _u64, _u64, _u64, _u64, _u32, _u64, _u32, _u32, _u64, _u64, _u64]),
+    "sz_matvec_cols_static": (_i32, [_i32, _u64, _u64, _u64, _u64, _u32, _u64, _u32, _u32, _u64]),
     "sz_session_new": (_vp, [C.POINTER(SessionConfig)]),
     "sz_session_free": (None, [_vp]),
     "sz_session_set_layer": (_i32, [_vp, _u32, _i32, _u64, _u64, _i32, _u64]),
@@ -439,6 +440,14 @@ def matvec_cols_scratch(ggml_type, cols, rows, m):
 
 def matvec_cols(ggml_type, w_dev, cols, rows, x_dev, xs, y_dev, ys, m, scratch=0, scratch_bytes=0, stream=0):
     check(lib().sz_matvec_cols(ggml_type, w_dev, cols, rows, x_dev, xs, y_dev, ys, m, scratch, scratch_bytes, stream))
+
+
+STATIC_WORKSPACE_BYTES = 4 << 20
+
+
+def matvec_cols_static(ggml_type, w_dev, cols, rows, x_dev, xs, y_dev, ys, m, stream=0):
+    """sz_matvec_cols on the library's own static device workspace: allocates nothing."""
+    check(lib().sz_matvec_cols_static(ggml_type, w_dev, cols, rows, x_dev, xs, y_dev, ys, m, stream))
 
 
 def verify_accept(ids, drafts):

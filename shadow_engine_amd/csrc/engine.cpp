@@ -112,7 +112,7 @@ static uint64_t cols_scratch_bytes(const Format& f, uint64_t cols, uint64_t rows
     return align16(ng * 8) + align16(ng * 17 * 4) + ng * exl3_ksplit((uint32_t) cols) * 4 * rows * 4;
 }
 
-static int matvec_cols_dev(int ty, uint64_t w, uint64_t cols, uint64_t rows, uint64_t x, uint32_t xs, uint64_t y, uint32_t ys, uint32_t m,
+int matvec_cols_dev(int ty, uint64_t w, uint64_t cols, uint64_t rows, uint64_t x, uint32_t xs, uint64_t y, uint32_t ys, uint32_t m,
                            uint64_t scratch, uint64_t scratch_bytes, uint64_t stream) {
     Format f;
     std::string tag;

@@ -39,13 +39,15 @@ static bool bind(void* lib, const char* name, F& fn, std::string& missing) {
     return fn != nullptr;
 }
 
+static void* g_hip_lib = nullptr;   // the bound libamdhip64, for the registration forwarders below
+
 HipApi& hip() {
     static HipApi api;
     static std::once_flag once;
     std::call_once(once, [] {
         std::string tried;
         // never unloaded, like the reference's libraries (dylib.rs:19-20)
-        void* lib = open_first("SHADOWZERO_HIP_LIB", {"libamdhip64.so", "libamdhip64.so.7", "libamdhip64.so.6", "/opt/rocm/lib/libamdhip64.so"}, tried);
+        void* lib = g_hip_lib = open_first("SHADOWZERO_HIP_LIB", {"libamdhip64.so", "libamdhip64.so.7", "libamdhip64.so.6", "/opt/rocm/lib/libamdhip64.so"}, tried);
         if (!lib) {
             api.error = "libamdhip64 not found (tried " + tried + ")";
             return;
@@ -100,6 +102,11 @@ HipApi& hip() {
         api.ok = true;
     });
     return api;
+}
+
+void* hip_symbol(const char* name) {
+    hip();
+    return g_hip_lib ? dlsym(g_hip_lib, name) : nullptr;
 }
 
 int hip_check(hipError_t e, const char* call) {
@@ -184,3 +191,33 @@ int rtc_compile(const char* name, const std::string& source, std::vector<char>& 
 }   // namespace sz
 
 extern "C" const char* sz_last_error(void) { return sz::last_error_cstr(); }
+
+// ---- what a hipcc-compiled translation unit of this library (csrc/static_workspace.hip: a `static __device__` array and
+// the host code that asks for its address) expects from the HIP runtime it would normally be linked against: the
+// registration of its device code at load time and two runtime calls.  They are forwarded to the library bound above, so
+// this library still links no ROCm library and there is one HIP runtime in the process; without libamdhip64 they do
+// nothing and the entry point that needs them reports it.  Hidden: nothing outside this library binds to them.
+extern "C" {
+#define SZ_HIDDEN __attribute__((visibility("hidden")))
+SZ_HIDDEN void** __hipRegisterFatBinary(const void* data) {
+    auto f = reinterpret_cast<void** (*)(const void*)>(sz::hip_symbol("__hipRegisterFatBinary"));
+    return f ? f(data) : nullptr;
+}
+SZ_HIDDEN void __hipRegisterVar(void** modules, void* var, char* host_name, char* device_name, int ext, size_t size, int constant, int global) {
+    auto f = reinterpret_cast<void (*)(void**, void*, char*, char*, int, size_t, int, int)>(sz::hip_symbol("__hipRegisterVar"));
+    if (f && modules) f(modules, var, host_name, device_name, ext, size, constant, global);
+}
+SZ_HIDDEN void __hipUnregisterFatBinary(void** modules) {
+    auto f = reinterpret_cast<void (*)(void**)>(sz::hip_symbol("__hipUnregisterFatBinary"));
+    if (f && modules) f(modules);
+}
+SZ_HIDDEN int hipGetSymbolAddress(void** dev_ptr, const void* symbol) {
+    auto f = reinterpret_cast<int (*)(void**, const void*)>(sz::hip_symbol("hipGetSymbolAddress"));
+    return f ? f(dev_ptr, symbol) : 1;   // hipErrorInvalidValue
+}
+SZ_HIDDEN int hipGetDevice(int* device) {
+    auto f = reinterpret_cast<int (*)(int*)>(sz::hip_symbol("hipGetDevice"));
+    return f ? f(device) : 1;
+}
+#undef SZ_HIDDEN
+}

@@ -300,6 +300,8 @@ int32_t sz_init(int32_t device) {
     if (load_programs()) return 1;
     g_device = device;
     g_init = true;
+    // the static workspace's address on this device (sz_matvec_cols_static); a failure is that entry point's to report
+    if (static_workspace_setup(device)) clear_error();
     return 0;
 }
 

@@ -71,6 +71,7 @@ struct HipApi {
 };
 HipApi& hip();                                  // binds on first use; hip().ok says whether it worked
 int hip_check(hipError_t e, const char* call);  // 0, or fail("call: name (string)")
+void* hip_symbol(const char* name);             // any other entry point of the bound libamdhip64 (nullptr: not there)
 
 // hiprtc, bound the same way (the nvrtc* table of crates/shadowzero-cuda/src/nvrtc.rs:21-37); optional.
 struct RtcApi {
@@ -143,5 +144,11 @@ bool format_of(int ggml_type, Format& f, std::string& tag_storage);
 uint64_t matrix_bytes(const Format& f, uint64_t cols, uint64_t rows);
 uint32_t rows_per_block(const Format& f, uint32_t cols, uint32_t cap = 64, uint32_t lds = 16384);   // rpb of the staged GGUF kernels (0: shape not supported by them)
 uint32_t exl3_ksplit(uint32_t in_f);
+// y_j = W x_j, j < m <= 8, on device addresses (sz_matvec_cols): launches only, nothing is allocated.
+int matvec_cols_dev(int ty, uint64_t w, uint64_t cols, uint64_t rows, uint64_t x, uint32_t xs, uint64_t y, uint32_t ys, uint32_t m, uint64_t scratch,
+                    uint64_t scratch_bytes, uint64_t stream);
+// The library's static device workspace (csrc/static_workspace.hip): its address on `device`, which must be current, is
+// looked up once and kept.  0 = ok.
+int static_workspace_setup(int device);
 
 }   // namespace sz
