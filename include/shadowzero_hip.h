@@ -200,6 +200,11 @@ int32_t sz_snapshot_download(const sz_snapshot*, uint32_t i, void* host, uint64_
  * range; uploads its table, runs and waits (the entries of copy_many_with, session.rs:3387). */
 int32_t sz_copy_ranges(const uint64_t* ranges, uint32_t n, uint64_t stream);
 
+/* The session's batch buffers, for tests and measurements (device addresses; the contents are those of the last call):
+ * 0 the plan (chosen experts u32[m][k], weights f32[m][k], counts u32[m] for the fused layers), 1 the split-k partial sums of
+ * gate and up, 2 the down products.  0 for any other `which`. */
+uint64_t sz_session_buffer(sz_session*, int32_t which);
+
 /* A whole verify round over device-resident inputs: for every layer l the MoE block on u[l][m][hidden] with rl[l][m][ne]
  * and sgl[l][m] into y[l][m][hidden], then the head on head_u[m][hidden], arg-max and acceptance against drafts[m-1]
  * (device).  out[0] = keep, out[1] = bonus token, out[2..2+m) = ids (device, u32).  Captured into a HIP graph on first

@@ -136,6 +136,7 @@ _SIGNATURES = {
     "sz_exl3_codebook": (_i32, [_u64, _u64]),
     "sz_matvec_cols_scratch": (_u64, [_i32, _u64, _u64, _u32]),
     "sz_matvec_cols": (_i32, [_i32, _u64, _u64, _u64, _u64, _u32, _u64, _u32, _u32, _u64, _u64, _u64]),
+    "sz_session_buffer": (_u64, [_vp, _i32]),
     "sz_matvec_cols_static": (_i32, [_i32, _u64, _u64, _u64, _u64, _u32, _u64, _u32, _u32, _u64]),
     "sz_session_new": (_vp, [C.POINTER(SessionConfig)]),
     "sz_session_free": (None, [_vp]),
@@ -481,6 +482,10 @@ class Session:
 
     def set_graph(self, enabled):
         check(lib().sz_session_set_graph(self._h, int(enabled)))
+
+    def buffer(self, which):
+        """Device address of a batch buffer: 0 plan, 1 gate/up partial sums, 2 down products."""
+        return lib().sz_session_buffer(self._h, which)
 
     def moe_layer_verify(self, layer, m, u_dev, rl_dev, sgl_dev, y_dev, stream=0):
         check(lib().sz_moe_layer_verify(self._h, layer, m, u_dev, rl_dev, sgl_dev, y_dev, stream))

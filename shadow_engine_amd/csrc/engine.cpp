@@ -612,6 +612,11 @@ int32_t sz_session_set_head(sz_session* s, int32_t ty, uint64_t w) {
     return 0;
 }
 
+uint64_t sz_session_buffer(sz_session* s, int32_t which) {
+    if (!s) return 0;
+    return which == 0 ? s->plan.ptr : which == 1 ? s->part.ptr : which == 2 ? s->dn.ptr : 0;
+}
+
 int32_t sz_session_set_graph(sz_session* s, int32_t enabled) {
     clear_error();
     if (!s) return fail("sz_session_set_graph: null session");

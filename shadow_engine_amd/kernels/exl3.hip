@@ -365,7 +365,7 @@ template <int K, bool H = false>
 __device__ __forceinline__ void exl3_grouped_kernel(const u64* __restrict__ wtab, const u32* __restrict__ gtab, const float* __restrict__ x, u32 xs,
                                                     float* __restrict__ part, u32 in_f, u32 out_f) {
     __shared__ float xw_all[4][4 * 128];
-    const u32 wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // the wave index as a scalar: the index arithmetic on it is the scalar unit's
     const u32 kb = blockIdx.z * 4 + wave;
     const u32* rec = gtab + 17 * (u64) blockIdx.y;
     const u32 n = min(rec[0], 4u);
@@ -490,7 +490,7 @@ __device__ __forceinline__ void verify_gate_up_kernel(const float* __restrict__ 
     __shared__ u32 s_top[16];
     static_assert(sizeof(wb_all) >= 512 * sizeof(double), "the exact routing fallback needs 512 doubles");
     const u32 G = m * k, S = G + m;
-    const u32 wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // the wave index as a scalar: the index arithmetic on it is the scalar unit's
     const u32 sel = blockIdx.y / S, pair = blockIdx.y % S;
     const u32 kbs = hidden / 128;
     const u32 kb0 = (blockIdx.z * WA + wave) * NB;
@@ -512,7 +512,11 @@ __device__ __forceinline__ void verify_gate_up_kernel(const float* __restrict__ 
     if (pair < G) {
         const u32 t = pair % k;
         if (wave == (blockIdx.x + blockIdx.y + blockIdx.z) % WA) {   // not always the same wave: the prologues of co-resident workgroups spread over the SIMDs
+            // the selection is a chain of dependent steps that the whole workgroup waits for: it goes ahead of the decoding
+            // waves of other workgroups on its SIMD
+            __builtin_amdgcn_s_setprio(3);
             route_id_of_rank(logits + (u64) j * ne, ne, k, t, lane, (double*) &wb_all[0][0], s_top);   // only s_top[t] is read
+            __builtin_amdgcn_s_setprio(0);
             if (sel == 0 && blockIdx.x == 0 && blockIdx.z == 0 && lane == 0) tidx[pair] = s_top[t];
         }
         __syncthreads();
@@ -578,7 +582,7 @@ __device__ __forceinline__ void verify_down_kernel(const float* __restrict__ log
     __shared__ float xw_all[4][128];
     __shared__ u32 sc_all[4][64];      // the wave's 128 f16 scales of down's inputs
     const u32 G = m * k, S = G + m;
-    const u32 wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // the wave index as a scalar: the index arithmetic on it is the scalar unit's
     const u32 pair = blockIdx.y;
     if (pair < G && pair % k == 0 && blockIdx.x == 0 && blockIdx.z == 0 && wave == 3) {
         // one wave a token: the routing weights and the count, for launch 3 (nothing in this launch reads them)

@@ -26,3 +26,17 @@ def exl3_k2_gate_proj():
     blob = np.fromfile(os.path.join(GOLDEN, "exl3_k2_gate_proj.blob"), np.uint8)
     assert blob.size == 2 * 2560 + 2 * 640 + 4 + 2560 * 640 * 2 // 8
     return 2560, 640, 2, blob
+
+
+def exl3_k4_shared_gate_proj():
+    """(in, out, K, blob) of the real K = 4 projection `layers.0.mlp.shared_expert.gate_proj` of the same fixture."""
+    blob = np.fromfile(os.path.join(GOLDEN, "exl3_k4_shared_gate_proj.blob"), np.uint8)
+    assert blob.size == 2 * 2560 + 2 * 640 + 4 + 2560 * 640 * 4 // 8
+    return 2560, 640, 4, blob
+
+
+def exl3_real_tensors():
+    """Both real tensors with what the reference recorded for them (crates/shadowzero-model/tests/exl3_vs_gguf.rs:133-134):
+    (in, out, K, blob, sum of squares, first four weights)."""
+    return [exl3_k2_gate_proj() + (287.702278, [-0.042833105, -0.0065446747, 0.029719023, -0.030945573]),
+            exl3_k4_shared_gate_proj() + (161.198363, [-0.0071623405, 0.00092289475, -0.0021615676, -0.0026322217])]

@@ -114,13 +114,13 @@ def test_exl3_half_rates_decode_bit_exact_and_multiply(gpu, bits_k):
         assert np.max(np.abs(ys[j] - want[j])) <= 2e-4 * np.max(np.abs(want[j]))
 
 
-def test_exl3_decode_of_the_real_tensor_is_bit_exact(gpu):
-    inf, outf, k, blob = golden_io.exl3_k2_gate_proj()
-    db = dev(gpu, blob)
-    out = gpu.empty(inf * outf, dtype=gpu.float32, device="cuda")
-    sz.dequantize(sz.EXL3(k), db.data_ptr(), out.data_ptr(), inf, outf)
-    gpu.cuda.synchronize()
-    assert np.array_equal(bits(out.cpu().numpy()), bits(O.exl3_reconstruct(inf, outf, k, blob, inner=True).ravel()))
+def test_exl3_decode_of_the_real_tensors_is_bit_exact(gpu):
+    for inf, outf, k, blob, _, _ in golden_io.exl3_real_tensors():      # K = 2 and K = 4
+        db = dev(gpu, blob)
+        out = gpu.empty(inf * outf, dtype=gpu.float32, device="cuda")
+        sz.dequantize(sz.EXL3(k), db.data_ptr(), out.data_ptr(), inf, outf)
+        gpu.cuda.synchronize()
+        assert np.array_equal(bits(out.cpu().numpy()), bits(O.exl3_reconstruct(inf, outf, k, blob, inner=True).ravel()))
 
 
 # ---------------------------------------------------------------------------------------------- Backend::matvec (B1)
@@ -160,12 +160,12 @@ def test_backend_matvec_exl3(gpu, bits_k, inf, outf):
     assert rel_l2(got, want) <= REL_L2
 
 
-def test_backend_matvec_on_the_real_exl3_tensor(gpu):
-    inf, outf, k, blob = golden_io.exl3_k2_gate_proj()
-    x = np.random.default_rng(5).normal(size=inf).astype(np.float32)
-    got = sz.GpuBackend().matvec(sz.EXL3(k), inf, outf, blob, "gate", x)
-    want = O.exl3_matvec(inf, outf, k, blob, x)
-    assert np.abs(got - want).max() <= 2e-4 * np.abs(want).max() and rel_l2(got, want) <= REL_L2
+def test_backend_matvec_on_the_real_exl3_tensors(gpu):
+    for inf, outf, k, blob, _, _ in golden_io.exl3_real_tensors():
+        x = np.random.default_rng(5).normal(size=inf).astype(np.float32)
+        got = sz.GpuBackend().matvec(sz.EXL3(k), inf, outf, blob, "gate%d" % k, x)
+        want = O.exl3_matvec(inf, outf, k, blob, x)
+        assert np.abs(got - want).max() <= 2e-4 * np.abs(want).max() and rel_l2(got, want) <= REL_L2
 
 
 def test_backend_refuses_what_it_cannot_run(gpu):
