@@ -197,7 +197,9 @@ int32_t sz_snapshot_take(sz_snapshot*, uint64_t stream);
 int32_t sz_snapshot_restore(sz_snapshot*, uint64_t stream);
 int32_t sz_snapshot_download(const sz_snapshot*, uint32_t i, void* host, uint64_t cap);
 /* The same launch for a one-off set: ranges[3 i ..] = (dst, src, bytes) device ranges, no destination overlapping another
- * range; uploads its table, runs and waits (the entries of copy_many_with, session.rs:3387). */
+ * range; uploads its table, runs and waits (the entries of copy_many_with, session.rs:3387).  It allocates and
+ * synchronizes the stream: it must not be called on a stream that is being captured (a snapshot object's take and
+ * restore are the forms that can be). */
 int32_t sz_copy_ranges(const uint64_t* ranges, uint32_t n, uint64_t stream);
 
 /* The session's batch buffers, for tests and measurements (device addresses; the contents are those of the last call):

@@ -459,9 +459,11 @@ int head_check(sz_session* s, uint32_t m, uint64_t u, const char* who) {
     return 0;
 }
 
+bool head_argmax_supported(const sz_session* s) { return s->head_type == SZ_TYPE_Q8_0; }
+
 int head_argmax(sz_session* s, uint32_t m, uint64_t u, uint64_t ids, uint64_t stream) {
     if (head_check(s, m, u, "sz_head_argmax")) return 1;
-    if (s->head_type != SZ_TYPE_Q8_0) return fail("sz_head_argmax: the fused head kernel is Q8_0 only");
+    if (!head_argmax_supported(s)) return fail("sz_head_argmax: the head's type has no fused arg-max kernel (Q8_0 or EXL3)");
     if (head_mfma_ok(s)) return head_argmax_mfma(s, m, u, 0, ids, stream);
     for (uint32_t j0 = 0; j0 < m; j0 += 4) {
         if (head_argmax_rows(s, std::min(4u, m - j0), u + (uint64_t) j0 * s->cfg.hidden * 4, 0, ids + j0 * 4ull, stream)) return 1;
@@ -707,6 +709,11 @@ int32_t sz_verify_round(sz_session* s, uint32_t m, uint64_t u, uint64_t rl, uint
     if (!s) return fail("sz_verify_round: null session");
     if (m == 0 || m > s->cfg.max_rows) return fail("sz_verify_round: " + std::to_string(m) + " rows");
     const sz_session_config& c = s->cfg;
+    // everything that can be refused is refused before a capture begins
+    if (head_check(s, m, head_u, "sz_verify_round")) return 1;
+    if (!head_argmax_supported(s)) return fail("sz_verify_round: the head's type has no fused arg-max kernel (Q8_0 or EXL3)");
+    for (uint32_t l = 0; l < c.n_layers; l++)
+        if (!s->layers[l].set) return fail("sz_verify_round: layer " + std::to_string(l) + " has no experts set");
     const SzGraphKey key{{m, u, rl, sgl, y, head_u, drafts, out, stream, 0}};
     auto it = s->use_graph ? s->graphs.find(key) : s->graphs.end();
     if (it == s->graphs.end()) {
@@ -726,7 +733,10 @@ int32_t sz_verify_round(sz_session* s, uint32_t m, uint64_t u, uint64_t rl, uint
         const std::string err = r ? sz_last_error() : "";
         uint64_t exec = 0;
         const int e = sz_capture_end(stream, &exec);
-        if (r) return fail(err);
+        if (r) {
+            if (!e && exec) sz_graph_destroy(exec);   // a graph of a round that could not be recorded is not kept
+            return fail(err);
+        }
         if (e) return 1;
         it = s->graphs.emplace(key, exec).first;
     }

@@ -852,9 +852,13 @@ extern "C" __global__ void __launch_bounds__(256) head_q8_0_argmax(const u8* w, 
 // The same head on the matrix cores, for cols <= 2048 (a multiple of 256), m <= 8 and a 16-byte aligned matrix.
 // A 16-row tile of the matrix (16 x cols / 32 x 34 contiguous bytes) comes into LDS by global-to-LDS loads, the next tile
 // while this one is multiplied.  Wave w owns the quarter k in [w cols / 4, (w + 1) cols / 4) of every row and keeps its
-// slice of the inputs in registers for the whole launch, as the B operands of v_mfma_f32_16x16x16_f16: column 2 j holds
-// f16(x_j), column 2 j + 1 holds f16(x_j - f16(x_j)), so the two columns together carry x_j to 22 bits and the product
-// with the int8 codes (exact in f16) is exact term by term; the matrix core adds in f32.  The A operand is the tile's
+// slice of the inputs in registers for the whole launch, as the B operands of v_mfma_f32_16x16x16_f16: with
+// s_j x_j = the input row times the power of two that takes its largest magnitude to [2^14, 2^15), column 2 j holds
+// f16(s_j x_j) and column 2 j + 1 holds f16(s_j x_j - f16(s_j x_j)): the high parts are finite whatever the activations'
+// size, the two columns together carry an element to 22 bits unless it is below 2^-17 of the row's largest (there the
+// low part runs into f16's subnormals and the element keeps at least its 11 high-part bits, an error below 2^-39 of
+// the largest), and every product with the int8 codes (exact in f16) is exact; the matrix core adds in f32 and the sums
+// are multiplied by 1 / s_j at the end.  The A operand is the tile's
 // codes: a lane takes 4 consecutive codes of row lane % 16, turns each into the f16 1024 + (code ^ 0x80) by putting 0x64
 // above the byte, and subtracts 1152 (exact).  A 32-block's two products are scaled by the block's f16 scale and added to
 // the lane's running sums in f32, block after block in k order; the four waves' sums are added in wave order.
@@ -894,6 +898,7 @@ extern "C" __global__ void __launch_bounds__(256, 2) head_q8_0_argmax_mfma(const
     __shared__ float red[4][256];
     __shared__ float s_bv[256];
     __shared__ u32 s_bi[256];
+    __shared__ float s_mx[4][8], s_inv[8];   // largest magnitude of a wave's quarter of every input row; the factor that undoes a row's scale
     const u32 tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const u32 rb = cols / 32 * 34, pitch = rb + 16;
     const u32 nbw = cols / 128;                           // 32-blocks of a wave's quarter of k (<= 16)
@@ -910,6 +915,24 @@ extern "C" __global__ void __launch_bounds__(256, 2) head_q8_0_argmax_mfma(const
         for (int b = 0; b < 16; b++)
 #pragma unroll
             for (int h = 0; h < 2; h++) raw[b][h] = *(const f32x4*) (xj + 32 * min((u32) b, nbw - 1) + 16 * h);
+        // every input row is scaled by a power of two that takes its largest magnitude to [2^14, 2^15) before it is split (the
+        // sums are scaled back at the end): the high parts cannot overflow to infinity whatever the activations' size, and
+        // the low parts of small activations are not lost to f16's subnormal range
+        float mxl = 0.0f;
+#pragma unroll
+        for (int b = 0; b < 16; b++)
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+                if ((u32) b < nbw)
+#pragma unroll
+                    for (int i = 0; i < 4; i++) mxl = fmaxf(mxl, __builtin_fabsf(raw[b][h][i]));   // a NaN is skipped here and shows in the sums
+        mxl = fmaxf(mxl, lane_xor<16>(mxl, lane));
+        mxl = fmaxf(mxl, lane_xor<32>(mxl, lane));
+        if (g4 == 0 && lowpart == 0) s_mx[wave][j] = mxl;
+        __syncthreads();
+        float scale, inv;
+        pow2_scale_of(f32_bits(fmaxf(fmaxf(s_mx[0][j], s_mx[1][j]), fmaxf(s_mx[2][j], s_mx[3][j]))), scale, inv);
+        if (wave == 0 && g4 == 0 && lowpart == 0) s_inv[j] = inv;
 #pragma unroll
         for (int b = 0; b < 16; b++)
 #pragma unroll
@@ -918,7 +941,7 @@ extern "C" __global__ void __launch_bounds__(256, 2) head_q8_0_argmax_mfma(const
                 if ((u32) b < nbw && j < m) {
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
-                        const float f = raw[b][h][i];
+                        const float f = raw[b][h][i] * scale;
                         const _Float16 hi = (_Float16) f;
                         v[i] = lowpart ? (_Float16) (f - (float) hi) : hi;
                     }
@@ -978,7 +1001,7 @@ extern "C" __global__ void __launch_bounds__(256, 2) head_q8_0_argmax_mfma(const
             const float o = lane_xor<1>(s, lane);
             const u32 n = tid & 15, j = n >> 1, row = 16 * t + (tid >> 4);
             if ((n & 1) == 0 && j < m && row < rows) {
-                float v = s + o;
+                float v = (s + o) * s_inv[j];
                 if (logits) logits[(u64) j * ls + row] = v;
                 if (v != v) v = -__builtin_inff();
                 argmax_merge(bv, bi, v, row);

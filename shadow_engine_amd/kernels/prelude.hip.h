@@ -81,6 +81,16 @@ __device__ __forceinline__ void argmax_merge(float& bv, u32& bi, float v, u32 i)
     }
 }
 
+// The power of two that takes a largest magnitude (the bits of a non-negative float) to [2^14, 2^15), and its inverse:
+// values scaled by it split into an f16 high part that cannot overflow and an f16 low part that keeps its bits down to
+// 2^-39 of the largest; a largest magnitude of zero, infinity or NaN gives 1.
+__device__ __forceinline__ void pow2_scale_of(u32 mx_bits, float& scale, float& inv) {
+    const u32 eb = (mx_bits >> 23) & 0xffu;
+    const u32 sb = (eb == 0u || eb == 255u) ? 127u : min(268u - eb, 253u);
+    scale = bits_f32(sb << 23);
+    inv = bits_f32((254u - sb) << 23);
+}
+
 // ---- global-to-LDS loads ------------------------------------------------------------------------------------------------
 // Written as inline assembly on purpose: the compiler then keeps no count of them, so it does not hold back the first LDS
 // read that follows until every one of them has landed; wait_vm is the only thing that orders them.  Consequences for the
