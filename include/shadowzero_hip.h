@@ -148,7 +148,10 @@ void sz_session_free(sz_session*);
  * one type; `shared` (0: none) is the shared expert in the same layout and of type shared_type. */
 int32_t sz_session_set_layer(sz_session*, uint32_t layer, int32_t expert_type, uint64_t experts, uint64_t stride, int32_t shared_type,
                              uint64_t shared);
-int32_t sz_session_set_head(sz_session*, int32_t ggml_type, uint64_t w);     /* output.weight, vocab x hidden */
+/* output.weight, vocab x hidden: Q8_0 or IQ3_S rows, or an EXL3 blob at a whole bit rate (in = hidden, out = vocab, both
+ * multiples of 128; the head of an EXL3 checkpoint, session.rs:7179-7187).  The fused arg-max (sz_head_argmax,
+ * sz_verify_round) exists for Q8_0 and EXL3; logits and the top 64 for all three. */
+int32_t sz_session_set_head(sz_session*, int32_t ggml_type, uint64_t w);
 /* 0: sz_verify_round launches its kernels one by one instead of replaying a captured graph (default 1). */
 int32_t sz_session_set_graph(sz_session*, int32_t enabled);
 /* moe_batch_resident (session.rs:8222): y[m][hidden] = the MoE block of layer l on u[m][hidden], from the router logits

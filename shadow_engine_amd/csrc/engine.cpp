@@ -295,6 +295,7 @@ struct sz_session {
     uint64_t head_w = 0;
     // batch buffers (session.rs `bb`): the plan, the expert products, the split-k partials, the head's scratch
     DevBuf plan, eg, act, eo, part, dn, head_part, logits, topv, topi, topo, ids;
+    DevBuf head_xa, head_inv;   // an EXL3 head's rotated inputs as f16 high and low parts (16 rows of 128 a 128-block), and the tokens' scales
     DevBuf rl, sgl;   // the router's outputs for a batch: f32[max_rows][n_expert], f32[max_rows]
     struct {
         DevBuf xq, xd, tidx, w, cnt, offs, list, items, hq, hd, eo;
@@ -459,11 +460,31 @@ int head_check(sz_session* s, uint32_t m, uint64_t u, const char* who) {
     return 0;
 }
 
-bool head_argmax_supported(const sz_session* s) { return s->head_type == SZ_TYPE_Q8_0; }
+bool head_is_exl3(const sz_session* s) { return s->head_type >= 1021 && s->head_type <= 1028; }
+bool head_argmax_supported(const sz_session* s) { return s->head_type == SZ_TYPE_Q8_0 || head_is_exl3(s); }
+
+// An EXL3 head (kernels/exl3.cu:349-461, 610-625 of the reference: rotate the rows once, then one pass over the matrix for all
+// m <= 8 rows): the arg-max ids (0: not wanted) and / or the logits (0: not written).
+int head_exl3(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uint64_t ids, uint64_t stream) {
+    const sz_session_config& c = s->cfg;
+    const uint32_t kbs = c.hidden / 128, bits = (uint32_t) s->head_type - 1020;
+    {
+        const sz_arg a[] = {P(s->head_w), P(u), U32(c.hidden), P(s->head_xa.ptr), P(s->head_inv.ptr), U32(c.hidden)};
+        if (launch("exl3_head_rotate", m, 1, 1, 64 * std::min<uint32_t>(16, kbs), 0, stream, a)) return 1;
+    }
+    const uint32_t nparts = c.vocab / 128, lds = 4 * ((kbs + 3) / 4) * ((m + 1) / 2) * 1024;
+    const std::string kn = "head_exl3_" + std::to_string(bits);
+    const sz_arg a[] = {P(s->head_w), P(s->head_xa.ptr), P(s->head_inv.ptr), P(logits), U32(c.vocab), P(s->head_part.ptr), U32(c.hidden), U32(c.vocab), U32(m)};
+    if (launch(kn.c_str(), nparts, 1, 1, 256, lds, stream, a)) return 1;
+    if (!ids) return 0;
+    const sz_arg b[] = {P(s->head_part.ptr), U32(nparts), U32(8), P(ids), P(0)};
+    return launch("argmax_merge_parts", m, 1, 1, 256, 0, stream, b);
+}
 
 int head_argmax(sz_session* s, uint32_t m, uint64_t u, uint64_t ids, uint64_t stream) {
     if (head_check(s, m, u, "sz_head_argmax")) return 1;
     if (!head_argmax_supported(s)) return fail("sz_head_argmax: the head's type has no fused arg-max kernel (Q8_0 or EXL3)");
+    if (head_is_exl3(s)) return head_exl3(s, m, u, 0, ids, stream);
     if (head_mfma_ok(s)) return head_argmax_mfma(s, m, u, 0, ids, stream);
     for (uint32_t j0 = 0; j0 < m; j0 += 4) {
         if (head_argmax_rows(s, std::min(4u, m - j0), u + (uint64_t) j0 * s->cfg.hidden * 4, 0, ids + j0 * 4ull, stream)) return 1;
@@ -473,6 +494,7 @@ int head_argmax(sz_session* s, uint32_t m, uint64_t u, uint64_t ids, uint64_t st
 
 int head_logits(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uint64_t stream) {
     if (head_check(s, m, u, "sz_head_logits")) return 1;
+    if (head_is_exl3(s)) return head_exl3(s, m, u, logits, 0, stream);
     const sz_session_config& c = s->cfg;
     return matvec_cols_dev(s->head_type, s->head_w, c.hidden, c.vocab, u, c.hidden, logits, c.vocab, m, 0, 0, stream);
 }
@@ -605,8 +627,14 @@ int32_t sz_moe_block_verify(sz_session* s, uint32_t l, uint32_t m, uint64_t u, u
 int32_t sz_session_set_head(sz_session* s, int32_t ty, uint64_t w) {
     clear_error();
     if (!s) return fail("sz_session_set_head: null session");
-    if (ty != SZ_TYPE_Q8_0 && ty != SZ_TYPE_IQ3_S) return fail("sz_session_set_head: the head must be Q8_0 or IQ3_S");
+    const bool exl3 = ty >= 1021 && ty <= 1028;
+    if (ty != SZ_TYPE_Q8_0 && ty != SZ_TYPE_IQ3_S && !exl3) return fail("sz_session_set_head: the head must be Q8_0, IQ3_S or EXL3 at a whole bit rate");
     if (w & 15) return fail("sz_session_set_head: the head must be 16-byte aligned");
+    if (exl3) {
+        const sz_session_config& c = s->cfg;
+        if (c.vocab == 0 || c.vocab % 128 || c.hidden % 128 || c.hidden > 8192) return fail("sz_session_set_head: an EXL3 head needs hidden (<= 8192) and the vocabulary to be multiples of 128");
+        if (s->head_xa.need((uint64_t) c.hidden / 128 * 16 * 256) || s->head_inv.need(64)) return 1;
+    }
     s->head_type = ty;
     s->head_w = w;
     for (auto& g : s->graphs) sz_graph_destroy(g.second);

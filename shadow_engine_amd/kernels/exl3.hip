@@ -794,6 +794,267 @@ extern "C" __global__ void __launch_bounds__(1024) verify_combine_exl3(const flo
     }
 }
 
+// ------------------------------------------------------------------------------------- the EXL3 head on the matrix cores
+// The lm_head of an EXL3 checkpoint (in = hidden, out = vocabulary; kernels/exl3.cu:349-461, 610-625: exl3_rotate_rows_f32 and
+// matvec_cols_exl3_pre of the reference) for the m <= 8 rows of a verify batch in one pass over the matrix, with the
+// arg-max fused in.  The dot products run on the matrix cores (v_mfma_f32_16x16x16_f16, one a 16 x 16 tile): operand B is
+// the tile, a lane supplying 4 CONSECUTIVE weights of the bit stream, which are input rows 2 a, 2 a + 1, 2 a + 8, 2 a + 9
+// (a = lane / 16) of output column lane % 16 (exl3.rs:106); their four 16-bit windows lie in the 16 + 3 K stream bits
+// that end at bit (t0 + 4) K, t0 = 32 (n % 8) + 8 a + 4 (n / 8): one funnel shift of two ring words (a per-lane constant
+// choice) brings them into a register and the windows are then at fixed shifts (two shifts for K > 5).  Operand A is the
+// input: row 2 j holds the f16 high part and row 2 j + 1 the f16 low part of token j's rotated input, scaled by the
+// power of two that takes the token's largest rotated magnitude to [2^14, 2^15), in the same k order: every product with
+// an f16 weight is exact, the matrix core adds in f32, and 8 tokens cost what one costs.
+typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
+
+// Where element q (0..15) of a tile row's 16 inputs sits in the row's 16 slots of an A row: lane group a reads the slots
+// 4 a .. 4 a + 3 = inputs 2 a, 2 a + 1, 2 a + 8, 2 a + 9 as one 8-byte word.
+__device__ __forceinline__ u32 exl3_aslot(u32 q) { return 4 * ((q & 7) >> 1) + 2 * (q >> 3) + (q & 1); }
+
+// Launch 1 of the head: token j = blockIdx.x.  Wave w rotates the 128-blocks w, w + waves, .. of x_j (x * suh, the
+// transform), the largest magnitude over the row gives the token's scale, and the scaled values go out as f16 high and
+// low parts: xa[(kb * 16 + 2 j + part) * 128 + 16 t8 + slot] for tile row t8 of block kb; inv[j] undoes the scale.
+// grid = m, block = 64 * min(16, in / 128).
+#define EXL3_HEAD_NB 4   /* 128-blocks a wave rotates at most: in <= 8192 */
+extern "C" __global__ void __launch_bounds__(1024) exl3_head_rotate(const u8* blob, const float* x, u32 xs, u16* xa, float* inv, u32 in_f) {
+    __shared__ float s_mx[16];
+    const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, nw = blockDim.x >> 6, j = blockIdx.x;
+    const u32 kbs = in_f / 128;
+    const u16* suh = (const u16*) blob;
+    float rot[EXL3_HEAD_NB][2];
+    float mx = 0.0f;
+#pragma unroll
+    for (int q = 0; q < EXL3_HEAD_NB; q++) {
+        const u32 kb = wave + nw * q;
+        rot[q][0] = rot[q][1] = 0.0f;
+        if (kb < kbs) {
+            const float* xj = x + (u64) j * xs + kb * 128;
+            float a0 = xj[lane] * f16_to_f32(suh[kb * 128 + lane]), a1 = xj[lane + 64] * f16_to_f32(suh[kb * 128 + 64 + lane]);
+            wht128_wave(a0, a1, lane);
+            rot[q][0] = a0;
+            rot[q][1] = a1;
+            mx = fmaxf(mx, fmaxf(__builtin_fabsf(a0), __builtin_fabsf(a1)));
+        }
+    }
+    mx = wave_max_f32(mx);
+    if (lane == 0) s_mx[wave] = mx;
+    __syncthreads();
+    float all = 0.0f;
+    for (u32 w = 0; w < nw; w++) all = fmaxf(all, s_mx[w]);
+    float scale, iv;
+    pow2_scale_of(f32_bits(all), scale, iv);
+    if (threadIdx.x == 0) inv[j] = iv;
+#pragma unroll
+    for (int q = 0; q < EXL3_HEAD_NB; q++) {
+        const u32 kb = wave + nw * q;
+        if (kb < kbs) {
+            u16* blk = xa + ((u64) kb * 16 + 2 * j) * 128;
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const u32 i = lane + 64 * h;
+                const float v = rot[q][h] * scale;
+                const _Float16 hi = (_Float16) v;
+                const _Float16 lo = (_Float16) (v - (float) hi);
+                const u32 at = 16 * (i >> 4) + exl3_aslot(i & 15);
+                blk[at] = __builtin_bit_cast(u16, hi);
+                blk[128 + at] = __builtin_bit_cast(u16, lo);
+            }
+        }
+    }
+}
+
+// Launch 2 of the head: output block ob = blockIdx.x (128 columns of the vocabulary).  Wave w of 4 takes the 128-blocks
+// w, w + 4, .. of the input (8 tile rows each) through a ring of 4 rows; its A rows (2 m rows of 128 f16 a block, copied
+// from xa once, in units of 4 rows) sit in LDS.  The four waves' sums are added in wave order, scaled back, taken through
+// the output-side transform and scales, optionally stored as logits[j * ls + column], and the block's best column of every
+// row goes to part[(ob * 8 + j) * 2] = {value bits, column} (a NaN counts as -inf, ties to the lower column).
+// grid = out / 128, block 256, dynamic LDS = 4 * ceil(in / 512) * ceil(m / 2) KiB.
+template <int K>
+__device__ __forceinline__ void exl3_head_kernel(const u8* __restrict__ blob, const u16* __restrict__ xa, const float* __restrict__ inv,
+                                                 float* __restrict__ logits, u32 ls, u32* __restrict__ part, u32 in_f, u32 out_f, u32 m) {
+    constexpr int D = 4;
+    typedef Exl3Rows<K, D> R;
+    constexpr int stride = R::stride, ur = R::unit_rows;
+    constexpr bool one_shift = 16 + 3 * K <= 32;
+    extern __shared__ __attribute__((aligned(16))) u16 a_sh[];            // [wave][its blocks][4 nq A rows][128]; afterwards the waves' sums
+    __shared__ __attribute__((aligned(16))) u32 wb_all[4][R::words];
+    const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, ob = blockIdx.x;
+    const u32 kbs = in_f / 128, nkbw = (kbs + 3) / 4, nq = (m + 1) / 2;
+    const u32 nkb = wave < kbs ? (kbs - wave + 3) / 4 : 0;                 // this wave's blocks: wave, wave + 4, ..
+    const u32 nr = nkb * 8;
+    const u32 nt = out_f / 16;
+    const u64 pitch = (u64) nt * EXL3_TILE_WORDS(K, false);
+    const u32* tr = (const u32*) (blob + 2 * (u64) in_f + 2 * (u64) out_f + 4) + (u64) ob * 8 * EXL3_TILE_WORDS(K, false);
+    const u32 wb_lds = __builtin_amdgcn_readfirstlane(lds_offset(wb_all[wave]));
+    u16* aw = a_sh + (u64) wave * nkbw * nq * 512;                        // 512 f16 = 1 KiB = 4 A rows
+    const u32 aw_lds = __builtin_amdgcn_readfirstlane(lds_offset(aw));
+    // relative row i of the wave is tile row (wave + 4 (i / 8)) * 8 + i % 8 of the matrix
+    auto row_ptr = [&](u32 i) -> const u32* { return tr + (u64) ((wave + 4 * (i >> 3)) * 8 + (i & 7)) * pitch; };
+    auto issue = [&](u32 i) {                   // the unit that starts at relative row i (a multiple of ur) into its ring slot
+        const u32 slot = i & (D - 1);
+        if constexpr (K == 4 || K == 3) {
+            lds_load<4 * K>(row_ptr(i) + lane * K, wb_lds + slot * 1024);
+        } else if constexpr (K == 2) {
+            lds_load<16>(row_ptr(i + (lane >> 5)) + (lane & 31) * 4, wb_lds + slot * 512);
+        } else {
+#pragma unroll
+            for (int d = 0; d < K; d++) lds_load<4>(row_ptr(i) + d * 64 + lane, wb_lds + slot * 256 * K + d * 256);
+        }
+    };
+    // the wave's A rows first (nq KiB a block), then its first rows
+    for (u32 kbl = 0; kbl < nkb; kbl++)
+        for (u32 qi = 0; qi < nq; qi++)
+            lds_load<16>((const u8*) xa + ((u64) (wave + 4 * kbl) * 16 + 4 * qi) * 256 + lane * 16, aw_lds + (kbl * nq + qi) * 1024);
+    u32 nring = 0;
+    for (u32 i = 0; i < (u32) D && i < nr; i += ur) {
+        issue(i);
+        nring += R::unit_loads;
+    }
+    // the A rows have landed once only the ring's loads are in flight (at most 4 K of them: K <= 8)
+    switch (nring) {
+        case 0: wait_vm<0>(); break;
+        case 1: wait_vm<1>(); break;
+        case 2: wait_vm<2>(); break;
+        case 3: wait_vm<3>(); break;
+        case 4: wait_vm<4>(); break;
+        case 5: wait_vm<5>(); break;
+        case 6: wait_vm<6>(); break;
+        case 7: wait_vm<7>(); break;
+        case 8: wait_vm<8>(); break;
+        case 12: wait_vm<12>(); break;
+        case 16: wait_vm<16>(); break;
+        case 20: wait_vm<20>(); break;
+        case 24: wait_vm<24>(); break;
+        case 28: wait_vm<28>(); break;
+        case 32: wait_vm<32>(); break;
+        default: wait_vm<0>(); break;
+    }
+    const u32 n = lane & 15, a = lane >> 4;
+    const u32 t0 = 32 * (n & 7) + 8 * a + 4 * (n >> 3);
+    // the 32 stream bits that end at bit e (exclusive) of the tile's ring: word jp holds the last of them, word jm the rest
+    auto window = [&](u32 e, u32& om, u32& op, u32& sh) {
+        const u32 jp = (e - 1) >> 5, jm = (jp + 8 * K - 1) % (8 * K);
+        sh = 31 - ((e - 1) & 31);
+        om = (jm / K) * stride + jm % K;   // a tile's word j sits at decode lane j / K, word j % K of that lane
+        op = (jp / K) * stride + jp % K;
+    };
+    u32 om1, op1, sh1, om0 = 0, op0 = 0, sh0 = 0;
+    window((t0 + 4) * K, om1, op1, sh1);
+    if constexpr (!one_shift) window((t0 + 2) * K, om0, op0, sh0);
+    f32x4 acc[8];
+#pragma unroll
+    for (int c = 0; c < 8; c++) acc[c] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    const bool fed = n < 2 * m;                            // this lane supplies A row n
+    const u16* xa0 = aw + (fed ? n : 0) * 128 + 4 * a;
+    const u32* wb = wb_all[wave];
+#pragma unroll 1
+    for (u32 i = 0; i < nr; i++) {
+        exl3_rows_wait<K, D>(i + D > nr ? i + D - nr : 0);
+        const u32* row = wb + (i & (D - 1)) * R::row_words;
+        u32 w1[8][2], w0[8][2];
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            w1[c][0] = row[c * 8 * stride + om1];
+            w1[c][1] = row[c * 8 * stride + op1];
+            if constexpr (!one_shift) {
+                w0[c][0] = row[c * 8 * stride + om0];
+                w0[c][1] = row[c * 8 * stride + op0];
+            }
+        }
+        typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+        u32x2 xv = *(const u32x2*) (xa0 + (u64) (i >> 3) * nq * 512 + 16 * (i & 7));
+        if (!fed) xv = u32x2{0u, 0u};
+        // the row's words are in registers once the reads have returned: its slot can take the row D further on
+        if ((i + 1) % ur == 0 && i + D + 1 - ur < nr) {
+            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
+            issue(i + D + 1 - ur);
+        }
+        const f16x4 av = __builtin_bit_cast(f16x4, xv);
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            const u32 hi = __builtin_amdgcn_alignbit(w1[c][0], w1[c][1], sh1);
+            u32 s0, s1;
+            if constexpr (one_shift) {
+                s0 = __builtin_amdgcn_ubfe(hi, 3 * K, 16);
+                s1 = __builtin_amdgcn_ubfe(hi, 2 * K, 16);
+            } else {
+                const u32 lo = __builtin_amdgcn_alignbit(w0[c][0], w0[c][1], sh0);
+                s0 = __builtin_amdgcn_ubfe(lo, K, 16);
+                s1 = lo & 0xffffu;
+            }
+            const u32 s2 = __builtin_amdgcn_ubfe(hi, K, 16), s3 = hi & 0xffffu;
+            const f16x2 b01 = exl3_cb2_pair(s0, s1), b23 = exl3_cb2_pair(s2, s3);
+            const f16x4 bv = {b01[0], b01[1], b23[0], b23[1]};
+            acc[c] = __builtin_amdgcn_mfma_f32_16x16x16f16(av, bv, acc[c], 0, 0, 0);
+        }
+    }
+    __syncthreads();                                       // every wave is done with its A rows: the space takes the sums
+    // D rows 4 a + i: lane group a holds tokens 2 a and 2 a + 1 (high part + low part each); red[wave][token][128]
+    float* red = (float*) a_sh;
+    {
+        float* o = red + (u64) wave * m * 128;
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            if (2 * a < m) o[(2 * a) * 128 + 16 * c + n] = acc[c][0] + acc[c][1];
+            if (2 * a + 1 < m) o[(2 * a + 1) * 128 + 16 * c + n] = acc[c][2] + acc[c][3];
+        }
+    }
+    __syncthreads();
+    const u16* svh = (const u16*) (blob + 2 * (u64) in_f) + ob * 128;
+    const float sv0 = f16_to_f32(svh[lane]), sv1 = f16_to_f32(svh[lane + 64]);
+    for (u32 j = wave; j < m; j += 4) {
+        float v0 = 0.0f, v1 = 0.0f;
+        for (u32 w = 0; w < 4; w++) {
+            v0 += red[((u64) w * m + j) * 128 + lane];
+            v1 += red[((u64) w * m + j) * 128 + lane + 64];
+        }
+        const float iv = inv[j];
+        v0 *= iv;
+        v1 *= iv;
+        wht128_wave(v0, v1, lane);
+        v0 *= sv0;
+        v1 *= sv1;
+        const u32 c0 = ob * 128 + lane, c1 = c0 + 64;
+        if (logits) {
+            logits[(u64) j * ls + c0] = v0;
+            logits[(u64) j * ls + c1] = v1;
+        }
+        float bv = v0 != v0 ? -__builtin_inff() : v0;
+        u32 bi = c0;
+        argmax_merge(bv, bi, v1 != v1 ? -__builtin_inff() : v1, c1);
+#pragma unroll
+        for (int h = 1; h < 64; h <<= 1) {
+            float ov;
+            u32 oi;
+            if (h == 1) { ov = lane_xor<1>(bv, lane); oi = f32_bits(lane_xor<1>(bits_f32(bi), lane)); }
+            else if (h == 2) { ov = lane_xor<2>(bv, lane); oi = f32_bits(lane_xor<2>(bits_f32(bi), lane)); }
+            else if (h == 4) { ov = lane_xor<4>(bv, lane); oi = f32_bits(lane_xor<4>(bits_f32(bi), lane)); }
+            else if (h == 8) { ov = lane_xor<8>(bv, lane); oi = f32_bits(lane_xor<8>(bits_f32(bi), lane)); }
+            else if (h == 16) { ov = lane_xor<16>(bv, lane); oi = f32_bits(lane_xor<16>(bits_f32(bi), lane)); }
+            else { ov = lane_xor<32>(bv, lane); oi = f32_bits(lane_xor<32>(bits_f32(bi), lane)); }
+            argmax_merge(bv, bi, ov, oi);
+        }
+        if (lane == 0) {
+            part[((u64) ob * 8 + j) * 2] = f32_bits(bv);
+            part[((u64) ob * 8 + j) * 2 + 1] = bi;
+        }
+    }
+}
+
+#define EXL3_HEAD_ENTRIES(K)                                                                                                          \
+    extern "C" __global__ void __launch_bounds__(256) head_exl3_##K(const u8* blob, const u16* xa, const float* inv, float* logits, u32 ls, \
+                                                                     u32* part, u32 in_f, u32 out_f, u32 m) {                             \
+        exl3_head_kernel<K>(blob, xa, inv, logits, ls, part, in_f, out_f, m);                                                         \
+    }
+EXL3_HEAD_ENTRIES(1)
+EXL3_HEAD_ENTRIES(2)
+EXL3_HEAD_ENTRIES(3)
+EXL3_HEAD_ENTRIES(4)
+EXL3_HEAD_ENTRIES(5)
+EXL3_HEAD_ENTRIES(6)
+EXL3_HEAD_ENTRIES(7)
+EXL3_HEAD_ENTRIES(8)
+
 // The one-matrix plan of a plain y_j = W x_j product for m <= 8 inputs: groups of 4 inputs, input row = output row = j.
 // grid 1, block 64.
 extern "C" __global__ void __launch_bounds__(64) cols_plan(u64* wtab, u32* gtab, u64 w, u32 m) {

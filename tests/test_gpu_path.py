@@ -655,6 +655,145 @@ def test_head_on_very_large_and_very_small_activations(gpu, scale):
         assert np.array_equal(tids[:8], wi[:8]) and rel_l2(vals, wv) <= REL_L2
 
 
+def exl3_head_reference(blob, hidden, vocab, kb, u):
+    """The oracle's logits of an EXL3 head for every input row (exl3.rs:528-599 matvec_blob)."""
+    return [O.exl3_matvec(hidden, vocab, kb, blob, u[j]) for j in range(u.shape[0])]
+
+
+def clear_gap(v, rank=1):
+    """True when the `rank` largest values of v are further apart (relatively) than f32 summation noise can move them."""
+    top = np.sort(v)[-(rank + 1):][::-1]
+    return bool(np.all(top[:-1] - top[1:] > 1e-5 * np.abs(top[:-1])))
+
+
+@pytest.mark.parametrize("kb,m,hidden,vocab", [(1, 2, 256, 512), (2, 3, 512, 1024), (3, 1, 512, 1024), (3, 8, 512, 1024), (4, 5, 768, 640),
+                                              (5, 4, 512, 1024), (6, 7, 256, 512), (7, 2, 256, 256), (8, 8, 512, 1024), (4, 4, 2560, 1280)])
+def test_exl3_head_argmax_logits_and_top_64_match_the_oracle(gpu, kb, m, hidden, vocab):
+    """The lm_head of an EXL3 checkpoint (session.rs:7179-7187): fused arg-max ids bit-exact with the oracle's arg-max, logits
+    within the reference's 2e-4 max|y| (tests/exl3.rs:45), the top 64 in the oracle's order; any whole rate, 1..8 rows."""
+    rng = np.random.default_rng(1000 * kb + m)
+    blob = synth.exl3_blob(rng, hidden, vocab, kb)
+    u = rng.normal(size=(m, hidden)).astype(np.float32)
+    u[0] *= 1.0e5                                            # a row far beyond f16's range, and a tiny one
+    if m > 1:
+        u[1] *= 3.0e-6
+    db, du = dev(gpu, blob), dev(gpu, u)
+    s = sz.Session(hidden, 512, 8, 2, 0, vocab, 8)
+    s.set_head(sz.EXL3(kb), db.data_ptr())
+    ids = gpu.zeros(8, dtype=gpu.int32, device="cuda")
+    s.head_argmax(m, du.data_ptr(), ids.data_ptr())
+    logits = gpu.zeros((m, vocab), dtype=gpu.float32, device="cuda")
+    s.head_logits(m, du.data_ptr(), logits.data_ptr())
+    top = s.head_top(m, du.data_ptr())
+    gpu.cuda.synchronize()
+    got_ids, got = ids.cpu().numpy().astype(np.uint32)[:m], logits.cpu().numpy()
+    want = exl3_head_reference(blob, hidden, vocab, kb, u)
+    for j in range(m):
+        assert np.abs(got[j] - want[j]).max() <= 2e-4 * np.abs(want[j]).max() and rel_l2(got[j], want[j]) <= REL_L2
+        assert clear_gap(want[j]), "pick another seed: the oracle's two largest logits are within f32 noise"
+        assert got_ids[j] == O.argmax(want[j]) == O.argmax(got[j])
+        vals, tids = top[j]
+        wv, wi = O.topk(want[j])
+        assert np.array_equal(tids, O.topk(got[j])[1])      # the exact top 64 of the GPU's own logits, ties to the lower id
+        n_clear = 0
+        while n_clear < 64 and clear_gap(want[j], n_clear + 1):
+            n_clear += 1
+        assert n_clear >= 4 and np.array_equal(tids[:n_clear], wi[:n_clear]) and rel_l2(vals, wv) <= REL_L2
+
+
+def test_exl3_head_prefers_the_lowest_id_on_exact_ties(gpu):
+    """Two 128-column blocks of the head with the same tiles and output scales give the same logits column by column: the
+    lower column must win, also across the blocks' workgroups."""
+    rng = np.random.default_rng(9)
+    kb, hidden, vocab, m = 3, 512, 1024, 3
+    blob = synth.exl3_blob(rng, hidden, vocab, kb).copy()
+    svh = blob[2 * hidden:2 * hidden + 2 * vocab].view(np.float16)
+    tr = blob[2 * hidden + 2 * vocab + 4:].view(np.uint16).reshape(hidden // 16, vocab // 16, 16 * kb)
+    src, dst = 2, 5                                          # block 5 becomes a copy of block 2; both are made the loudest
+    tr[:, 8 * dst:8 * dst + 8] = tr[:, 8 * src:8 * src + 8]
+    svh[128 * src:128 * src + 128] *= np.float16(8.0)
+    svh[128 * dst:128 * dst + 128] = svh[128 * src:128 * src + 128]
+    u = rng.normal(size=(m, hidden)).astype(np.float32)
+    db, du = dev(gpu, blob), dev(gpu, u)
+    s = sz.Session(hidden, 512, 8, 2, 0, vocab, 8)
+    s.set_head(sz.EXL3(kb), db.data_ptr())
+    ids = gpu.zeros(8, dtype=gpu.int32, device="cuda")
+    s.head_argmax(m, du.data_ptr(), ids.data_ptr())
+    top = s.head_top(m, du.data_ptr())
+    gpu.cuda.synchronize()
+    got_ids = ids.cpu().numpy().astype(np.uint32)[:m]
+    for j in range(m):
+        want = O.exl3_matvec(hidden, vocab, kb, blob, u[j])
+        best = O.argmax(want)
+        assert 128 * src <= best < 128 * src + 128 and want[best] == want[best + 128 * (dst - src)]
+        assert got_ids[j] == best
+        assert top[j][1][0] == best and top[j][1][1] == best + 128 * (dst - src)
+
+
+@pytest.mark.parametrize("kb,m", [(3, 1), (4, 4), (5, 8)])
+def test_exl3_head_full_size(gpu, kb, m):
+    """151 936 x 2048 at K = 3, 4, 5 for 1, 4 and 8 rows: ids equal to the oracle's arg-max, the top 64 in its order."""
+    rng = np.random.default_rng(50 + kb)
+    hidden, vocab = 2048, 151936
+    blob = synth.exl3_blob(rng, hidden, vocab, kb)
+    u = rng.normal(size=(m, hidden)).astype(np.float32)
+    db, du = dev(gpu, blob), dev(gpu, u)
+    s = sz.Session(hidden, 512, 8, 2, 0, vocab, 8)
+    s.set_head(sz.EXL3(kb), db.data_ptr())
+    ids = gpu.zeros(8, dtype=gpu.int32, device="cuda")
+    print("exl3 head", kb, m, flush=True)
+    s.head_argmax(m, du.data_ptr(), ids.data_ptr())
+    gpu.cuda.synchronize()
+    top = s.head_top(m, du.data_ptr())
+    got_ids = ids.cpu().numpy().astype(np.uint32)[:m]
+    for j in range(m):
+        want = O.exl3_matvec(hidden, vocab, kb, blob, u[j])
+        assert clear_gap(want), "pick another seed: the oracle's two largest logits are within f32 noise"
+        assert got_ids[j] == O.argmax(want)
+        vals, tids = top[j]
+        wv, wi = O.topk(want)
+        assert tids[0] == wi[0] and rel_l2(vals, wv) <= REL_L2 and len(set(tids.tolist()) & set(wi.tolist())) >= 62
+
+
+def test_verify_round_with_an_exl3_head(gpu):
+    """A round of a model whose head is EXL3 too (the mixed-rate checkpoint's own): ids, accepted count and the graph replays."""
+    rng = np.random.default_rng(31)
+    hidden, ff, ne, k, vocab, m, kb = 512, 256, 8, 3, 1024, 4, 4
+    s = sz.Session(hidden, ff, ne, k, 1, vocab, 8)
+    dbuf, stride, blobs, sh = build_layer(gpu, rng, sz.EXL3(3), hidden, ff, ne, True)
+    s.set_layer(0, sz.EXL3(3), dbuf.data_ptr(), stride, sz.EXL3(3), dbuf.data_ptr() + ne * stride)
+    head = synth.exl3_blob(rng, hidden, vocab, kb)
+    dh = dev(gpu, head)
+    s.set_head(sz.EXL3(kb), dh.data_ptr())
+    u = rng.normal(size=(1, m, hidden)).astype(np.float32)
+    rl = rng.normal(size=(1, m, ne)).astype(np.float32)
+    sgl = rng.normal(size=(1, m)).astype(np.float32)
+    hu = rng.normal(size=(m, hidden)).astype(np.float32)
+    du, drl, dsgl, dhu = dev(gpu, u), dev(gpu, rl), dev(gpu, sgl), dev(gpu, hu)
+    want = [O.exl3_matvec(hidden, vocab, kb, head, hu[j]) for j in range(m)]
+    assert all(clear_gap(w) for w in want)
+    want_ids = np.array([O.argmax(w) for w in want], np.uint32)
+    drafts = want_ids[:m - 1].copy()
+    drafts[2] = (drafts[2] + 1) % vocab                      # two of the three drafts are accepted
+    dd = dev(gpu, drafts.astype(np.int32))
+    out = gpu.zeros(2 + 8, dtype=gpu.int32, device="cuda")
+    y = gpu.zeros((1, m, hidden), dtype=gpu.float32, device="cuda")
+    stream = sz.Stream()
+    for replay in range(3):
+        out.zero_()
+        gpu.cuda.synchronize()
+        s.verify_round(m, du.data_ptr(), drl.data_ptr(), dsgl.data_ptr(), y.data_ptr(), dhu.data_ptr(), dd.data_ptr(), out.data_ptr(), stream.handle)
+        stream.synchronize()
+        o = out.cpu().numpy().view(np.uint32)
+        assert np.array_equal(o[2:2 + m], want_ids) and o[0] == 3 and o[1] == want_ids[2]
+    # a head without a fused arg-max is refused before anything is captured
+    wq = synth.iq3_s_matrix(rng, vocab, hidden)
+    dq = dev(gpu, wq)
+    s.set_head(sz.IQ3_S, dq.data_ptr())
+    with pytest.raises(sz.SzError, match="no fused arg-max"):
+        s.verify_round(m, du.data_ptr(), drl.data_ptr(), dsgl.data_ptr(), y.data_ptr(), dhu.data_ptr(), dd.data_ptr(), out.data_ptr(), stream.handle)
+
+
 def test_head_argmax_prefers_the_lowest_id_on_exact_ties(gpu):
     rng = np.random.default_rng(3)
     vocab, hidden = 640, 2048
