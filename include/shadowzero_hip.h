@@ -83,8 +83,13 @@ int32_t sz_ktime_begin(const char* prefix);
 int32_t sz_ktime_entry(int32_t i, const char** name, uint64_t* launches, double* total_ms);
 int32_t sz_ktime_end(void);
 /* The cache key (64 hex digits + NUL into `hex65`) of kernel file `file`: SHA-256 over the assembled source, the compile
- * options and the target, as nvrtc.rs:185-194.  Needs no device. */
+ * options, the target and the way it is built, as nvrtc.rs:185-194.  sz_program_cache_key names the object that hipcc
+ * builds ahead of time with sz_program_aot_options(file) (the library's options plus the file's `// hipcc:` lines),
+ * sz_program_cache_key_rtc the one the library compiles itself with hiprtc on a cache miss (the library's options only): the
+ * two are different binaries and never share a name.  Need no device. */
 int32_t sz_program_cache_key(const char* file, char* hex65);
+int32_t sz_program_cache_key_rtc(const char* file, char* hex65);
+const char* sz_program_aot_options(const char* file);
 int32_t sz_program_file_count(void);
 const char* sz_program_file_name(int32_t i);
 /* The directory code objects are cached in, and the compile options one `hipcc --genco` needs to fill it ahead of time

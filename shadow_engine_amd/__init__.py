@@ -121,6 +121,8 @@ _SIGNATURES = {
     "sz_ktime_entry": (_i32, [_i32, C.POINTER(C.c_char_p), C.POINTER(_u64), C.POINTER(C.c_double)]),
     "sz_ktime_end": (_i32, []),
     "sz_program_cache_key": (_i32, [C.c_char_p, C.c_char_p]),
+    "sz_program_cache_key_rtc": (_i32, [C.c_char_p, C.c_char_p]),
+    "sz_program_aot_options": (C.c_char_p, [C.c_char_p]),
     "sz_program_file_count": (_i32, []),
     "sz_program_file_name": (C.c_char_p, [_i32]),
     "sz_cache_dir": (C.c_char_p, []),

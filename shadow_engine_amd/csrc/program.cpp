@@ -130,11 +130,39 @@ int program_source(const char* file, std::string& out) {
     return 0;
 }
 
-int cache_key(const char* file, std::string& hex) {
+// The options a kernel file asks the ahead-of-time compiler for on top of compile_options(): its `// hipcc: <options>` lines,
+// joined by spaces (preferences of code generation; the run-time compiler does not get them).
+static std::string extra_options(const std::string& src) {
+    std::string out;
+    size_t pos = 0;
+    const std::string tag = "// hipcc: ";
+    while (pos < src.size()) {
+        size_t end = src.find('\n', pos);
+        if (end == std::string::npos) end = src.size();
+        if (src.compare(pos, tag.size(), tag) == 0) {
+            if (!out.empty()) out += ' ';
+            out += src.substr(pos + tag.size(), end - pos - tag.size());
+        }
+        pos = end + 1;
+    }
+    while (!out.empty() && (out.back() == ' ' || out.back() == '\r')) out.pop_back();
+    return out;
+}
+
+// The cache key of a kernel file's code object: SHA-256 over the assembled source, the options, the target and HOW it was
+// built (nvrtc.rs:185-194 hashes source + options + target).  An object compiled ahead of time by hipcc (with the file's extra
+// options) and one compiled at run time by hiprtc (without) are different binaries and get different names, so the one
+// can never stand in for the other.
+int cache_key(const char* file, std::string& hex, bool run_time) {
     std::string src;
     if (program_source(file, src)) return 1;
-    hex = sha256_hex(src + '\0' + compile_options() + '\0' + "gfx950");
+    const std::string opts = run_time ? std::string(compile_options()) : aot_options_of(src);
+    hex = sha256_hex(src + '\0' + opts + '\0' + "gfx950" + '\0' + (run_time ? "hiprtc" : "hipcc"));
     return 0;
+}
+std::string aot_options_of(const std::string& src) {
+    const std::string extra = extra_options(src);
+    return extra.empty() ? std::string(compile_options()) : std::string(compile_options()) + " " + extra;
 }
 
 // ---- loading and launching ----------------------------------------------------------------------------------------
@@ -169,14 +197,16 @@ static int load_file(int fi) {
     if (L.tried) return fail(L.error);
     L.tried = true;
     const char* file = SZ_FILES[fi];
-    std::string key;
-    if (cache_key(file, key)) {
+    std::string key, rkey;
+    if (cache_key(file, key, false) || cache_key(file, rkey, true)) {
         L.error = sz_last_error();
         return 1;
     }
-    const std::string path = cache_dir() + "/" + key + ".hsaco";
+    // the object built ahead of time first, then one an earlier run compiled with hiprtc
+    std::string path = cache_dir() + "/" + key + ".hsaco";
     std::string image;
-    if (!read_file(path, image)) {
+    if (!read_file(path, image)) path = cache_dir() + "/" + rkey + ".hsaco";
+    if (image.empty() && !read_file(path, image)) {
         // miss: compile at run time and fill the cache (tmp + rename; a failed write is tolerated, nvrtc.rs:247-254)
         std::string src, log;
         std::vector<char> code;
@@ -509,9 +539,24 @@ int32_t sz_ktime_end(void) {
 int32_t sz_program_cache_key(const char* file, char* hex65) {
     clear_error();
     std::string hex;
-    if (cache_key(file, hex)) return 1;
+    if (cache_key(file, hex, false)) return 1;
     std::memcpy(hex65, hex.c_str(), 65);
     return 0;
+}
+int32_t sz_program_cache_key_rtc(const char* file, char* hex65) {
+    clear_error();
+    std::string hex;
+    if (cache_key(file, hex, true)) return 1;
+    std::memcpy(hex65, hex.c_str(), 65);
+    return 0;
+}
+const char* sz_program_aot_options(const char* file) {
+    clear_error();
+    static thread_local std::string s;
+    std::string src;
+    if (program_source(file, src)) return nullptr;
+    s = aot_options_of(src);
+    return s.c_str();
 }
 int32_t sz_program_file_count(void) { return file_count(); }
 const char* sz_program_file_name(int32_t i) { return file_name(i); }

@@ -106,7 +106,8 @@ std::string kernel_dir();
 std::string cache_dir();
 const char* compile_options();
 int program_source(const char* file, std::string& out);   // prelude + headers + file
-int cache_key(const char* file, std::string& hex);
+int cache_key(const char* file, std::string& hex, bool run_time);   // of the object hipcc builds ahead of time, or of the one hiprtc builds
+std::string aot_options_of(const std::string& assembled_source);    // compile_options() + the file's `// hipcc:` lines
 std::string sha256_hex(const std::string& data);
 
 bool initialized();

@@ -52,15 +52,19 @@ def test_parse_param_vocabulary():
         build.parse_param("double z")
 
 
-def test_cache_key_is_sha256_of_source_options_and_target():
+def test_cache_key_is_sha256_of_source_options_target_and_build_mode():
+    """nvrtc.rs:185-194 hashes source + options + target; here also how the object is built: the one hipcc makes ahead of time
+    (with the file's own `// hipcc:` options) and the one hiprtc makes on a cache miss never share a name."""
     L = sz.lib()
     opts = L.sz_compile_options()
+    assert b"ffp-contract=off" in opts and b"packed-fp32-ops" in opts
+    extras = 0
     for i in range(L.sz_program_file_count()):
         name = L.sz_program_file_name(i)
         if not os.path.exists(os.path.join(build.KERNELS, name.decode())):
             continue
-        key = C.create_string_buffer(65)
-        assert L.sz_program_cache_key(name, key) == 0
+        key, rkey = C.create_string_buffer(65), C.create_string_buffer(65)
+        assert L.sz_program_cache_key(name, key) == 0 and L.sz_program_cache_key_rtc(name, rkey) == 0
         tmp = os.path.join(ROOT, "tests", ".src_probe.tmp")
         try:
             assert L.sz_program_write_source(name, tmp.encode()) == 0
@@ -68,8 +72,14 @@ def test_cache_key_is_sha256_of_source_options_and_target():
         finally:
             if os.path.exists(tmp):
                 os.remove(tmp)
-        assert key.value.decode() == hashlib.sha256(src + b"\0" + opts + b"\0gfx950").hexdigest()
-        assert b"ffp-contract=off" in opts and b"packed-fp32-ops" in opts
+        own = b" ".join(l[len(b"// hipcc: "):].strip() for l in src.split(b"\n") if l.startswith(b"// hipcc: "))
+        aot = L.sz_program_aot_options(name)
+        assert aot == (opts + b" " + own if own else opts)
+        extras += bool(own)
+        assert key.value.decode() == hashlib.sha256(src + b"\0" + aot + b"\0gfx950\0hipcc").hexdigest()
+        assert rkey.value.decode() == hashlib.sha256(src + b"\0" + opts + b"\0gfx950\0hiprtc").hexdigest()
+        assert key.value != rkey.value
+    assert extras >= 1          # prefill.hip asks for matrix results in vector registers
     key = C.create_string_buffer(65)
     assert L.sz_program_cache_key(b"nope.hip", key) != 0 and "not a registered kernel file" in sz.last_error()
 

@@ -969,6 +969,39 @@ def test_hiprtc_compiles_a_kernel_with_the_library_options(gpu):
     assert r != 0 and "error" in sz.last_error()          # the compile log comes back whole (nvrtc.rs:225-227)
 
 
+def test_the_library_compiles_its_own_kernel_files_at_run_time_in_a_fresh_process(gpu, tmp_path):
+    """kernels.rs:532-545, nvrtc.rs:180-256: with an empty code-object cache sz_init compiles all four kernel files with hiprtc
+    (global-to-LDS loads and wait counts in inline assembly, permlane swaps, matrix instructions), fills the cache under the
+    run-time keys, which are not the keys of the objects built ahead of time, and the smoke round (EXL3 layer, Q8_0 head,
+    arg-max, acceptance, against the oracle) passes on those objects."""
+    import os
+    import subprocess
+    import sys
+    import time
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    env = dict(os.environ, SHADOWZERO_KERNEL_CACHE=str(tmp_path))
+    t0 = time.time()
+    p = subprocess.Popen([sys.executable, "-u", "-c", "import __graft_entry__ as g; g.smoke()"], cwd=root, env=env,
+                         stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    while p.poll() is None:
+        time.sleep(5)
+        print("run-time compile: %.0f s" % (time.time() - t0), flush=True)
+    out = p.stdout.read()
+    assert p.returncode == 0 and "smoke ok" in out, out[-3000:]
+    import ctypes as C
+    lib = sz.lib()
+    made = sorted(f for f in os.listdir(tmp_path) if f.endswith(".hsaco"))
+    rtc, aot = [], []
+    for i in range(lib.sz_program_file_count()):
+        name = lib.sz_program_file_name(i)
+        k1, k2 = C.create_string_buffer(65), C.create_string_buffer(65)
+        assert lib.sz_program_cache_key_rtc(name, k1) == 0 and lib.sz_program_cache_key(name, k2) == 0
+        rtc.append(k1.value.decode() + ".hsaco")
+        aot.append(k2.value.decode() + ".hsaco")
+    assert made == sorted(rtc) and not set(rtc) & set(aot)
+    print("run-time compile of %d kernel files + smoke: %.0f s" % (len(made), time.time() - t0), flush=True)
+
+
 # ------------------------------------------------------------------------------------------- the int8 prefill chunk
 def test_activation_quantization_on_the_gpu_is_bit_exact(gpu):
     rng = np.random.default_rng(31)
