@@ -13,10 +13,16 @@ lines carry the same fields):
     config2  one IQ3_S MoE layer for one token (512 experts + shared, top-10); a step walks through 8 different layers
     config3  one EXL3 K=3 MoE layer for 4 tokens + head + acceptance (weights of the one layer stay warm in cache)
     config4  one prefill chunk: 512 tokens through the 512 IQ3_S experts of a layer on int8 activations (int8 MFMA)
+    exl3head the 151,936 x 2048 lm_head of an EXL3 checkpoint (--bits K, default 4) for the batch, arg-max fused in
     stage    one EXL3 layer of a safetensors checkpoint staged into HBM (the loader beside the path; PCIe-inclusive)
     snapshot the rollback point of a pass: 73 device ranges (79 MB of recurrent state) saved and put back, a launch each
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload config5] [--layers 48]
+
+The default run then times configurations 1-4 once each (`other_configs`).  `roofline` sets the dominant kernel against the
+HBM roof and, from the hardware counters in profiles/counters.json (quoted only while the kernel file they were measured on is
+unchanged), against the vector-ALU roof; `bound` names the nearer one.  `cpu_baseline` times the CPU oracle on one thread
+and on all hardware threads, best of 20 runs.
 """
 import argparse
 import json
@@ -32,39 +38,29 @@ sys.path.insert(0, ROOT)
 HBM_PEAK_GBPS = 8000.0
 INT8_MFMA_PEAK_TOPS = 5000.0
 HIDDEN, FF, NE, TOPK, VOCAB, ROWS = 2048, 512, 512, 10, 151936, 4
-# HBM bytes per launch (fetched + written) of the kernels of the default workload, from the memory counters of the
-# profile profiles/verify_round_config5_hbm_traffic.txt (FETCH_SIZE and WRITE_SIZE, each scaled by what the plain copy launch
-# of the same run reads).
-MEASURED_TRAFFIC = {
-    "head_q8_0_argmax_mfma": 331100287,
-    "verify_down_exl3_2": 19692128,
-    "verify_down_exl3_3": 25137765,
-    "verify_down_exl3_4": 30443937,
-    "verify_gate_up_exl3_2": 29546458,
-    "verify_gate_up_exl3_3": 40794359,
-    "verify_gate_up_exl3_4": 51646447,
-}
+COUNTERS = os.path.join(ROOT, "profiles", "counters.json")
+SIMDS = 256 * 4                                  # 256 compute units x 4 SIMDs; a wave64 vector instruction takes one for 4 cycles
 
 
-# Vector-ALU instructions (wave64) per launch of the same kernels at 4 rows, from profiles/verify_round_config5_valu_counters.txt
-# (SQ_INSTS_VALU).  The EXL3 decode is bound by these, not by HBM: a SIMD issues one such instruction in 4 cycles.
-MEASURED_VALU = {
-    "head_q8_0_argmax_mfma": 15415352,
-    "verify_down_exl3_2": 4118620,
-    "verify_down_exl3_3": 4146780,
-    "verify_down_exl3_4": 4158044,
-    "verify_gate_up_exl3_2": 8454992,
-    "verify_gate_up_exl3_3": 8477520,
-    "verify_gate_up_exl3_4": 8505680,
-}
-VALU_PEAK_GINST = 256 * 4 * 2.4 / 4          # 256 CUs x 4 SIMDs, one wave64 vector instruction in 4 cycles at 2.4 GHz: 614.4 G/s
+def load_counters(sz):
+    """profiles/counters.json (written by `python -m shadow_engine_amd.profile_counters` from rocprofv3 databases): per-kernel
+    hardware counters of the benchmark's workloads, stamped with the cache keys of the kernel files they were measured on.
+    Returns (counters or None, stale): stale maps every kernel whose file has changed since (or every kernel, when the
+    file is missing) to the reason its counters are not quoted."""
+    file_of = {name: f for name, f, _ in sz.kernels()}
+    try:
+        c = json.load(open(COUNTERS))
+    except (OSError, ValueError) as e:
+        return None, {k: "no usable profiles/counters.json (%s)" % type(e).__name__ for k in file_of}
+    now, then = sz.program_keys(), c.get("kernel_keys", {})
+    changed = sorted(f for f in now if then.get(f) != now[f])
+    return c, {k: "profiles/counters.json was measured on another %s" % f for k, f in file_of.items() if f in changed}
 
 
 class Workload:
     """step(): one pass, launched on `stream`; set_eager(bool): graph replay off/on where the workload has one;
     step_bytes: algorithmic bytes of a step; kernel_bytes: {kernel: algorithmic bytes per launch}; check(): raises if the
     pass went wrong; describe: the config object of the JSON line."""
-    traffic = {}
     extra = {}
     kernel_ops = {}
     cold_variant = False
@@ -134,14 +130,14 @@ def exl3_round(torch, sz, synth, synth_device, stream, L, rates, tag):
         w.kernel_bytes["verify_down_exl3_%d" % kb] = n_sel[kb] * dn_bytes[kb] + act_dn
     w.step, w.check, w.set_eager = step, check, (lambda eager: sess.set_graph(not eager))
     w.step_bytes = moe_bytes + head_bytes + act_bytes
-    w.traffic = MEASURED_TRAFFIC if (L == 48 and tag == "config 5" and ROWS == 4) else {}
+    w.counters_key = "config5" if (L == 48 and tag == "config 5" and ROWS == 4) else ("config3" if (tag == "config 3" and ROWS == 4) else None)
     w.cold_variant = tag == "config 3"
     w.dtype = "f32 accumulate over EXL3 f16 codebook weights / Q8_0 int8"
     w.describe = {"workload": "%s: verify round, %d MoE layer%s (hidden 2048, 512 experts + shared, top-10, EXL3 K in %s), %d-token batch, "
                               "Q8_0 lm_head 151936x2048, arg-max, greedy acceptance of %d drafts" % (tag, L, "s" if L > 1 else "", sorted(set(rates)), ROWS, ROWS - 1),
                   "layers": L, "rows": ROWS, "resident_GB": round(sum(b.numel() for b, _ in layers) / 1e9 + head.numel() / 1e9, 2)}
     w.extra = {"accepted_drafts": wrong}
-    w.cpu_args = (layers[0], rates[0], rl_h[0], u[0].cpu().numpy(), sgl[0].cpu().numpy())
+    w.cpu = ("exl3_token", (layers[0], rates[0], rl_h[0], u[0].cpu().numpy(), sgl[0].cpu().numpy()))
     w.keep = (sess, layers, head, u, rl, sgl, hu, y, out, drafts)
     return w
 
@@ -160,6 +156,7 @@ def q8_matvec(torch, sz, synth, synth_device, stream):
     w.dtype = "f32 accumulate over Q8_0 int8"
     w.cold_variant = True
     w.describe = {"workload": "config 1: Q8_0 1024x2048 matrix-vector product, one input (the matrix stays warm in cache between steps)"}
+    w.cpu = ("q8_0_matvec", (mat.cpu().numpy(), x.cpu().numpy(), rows, cols))
     w.keep = (mat, x, y)
     return w
 
@@ -195,6 +192,8 @@ def iq3s_decode(torch, sz, synth, synth_device, stream, L=8):
     w.describe = {"workload": "config 2: IQ3_S MoE layer for one token (hidden 2048, 512 experts + shared, top-10); a step is %d "
                               "different layers one after the other" % L, "layers": L, "rows": 1,
                   "resident_GB": round(sum(b.numel() for b in layers) / 1e9, 2)}
+    w.counters_key = "config2" if L == 8 else None
+    w.cpu = ("iq3_s_token", (layers[0], stride, rl[0].cpu().numpy(), u[0].cpu().numpy(), sgl[0].cpu().numpy()))
     w.keep = (sess, layers, u, rl, sgl, y)
     return w
 
@@ -223,7 +222,32 @@ def iq3s_prefill(torch, sz, synth, synth_device, stream, tokens=512):
     w.describe = {"workload": "config 4: prefill chunk, %d tokens x hidden 2048 through 512 IQ3_S experts (top-10, Zipf-skewed routing, "
                               "%d distinct experts hit) on per-32 int8 activations" % (tokens, distinct), "rows": tokens,
                   "resident_GB": round(buf.numel() / 1e9, 2)}
+    w.counters_key = "config4" if tokens == 512 else None
+    w.cpu = ("iq3_s_int8_pairs", (buf, stride, ids, x[:8].cpu().numpy()))
     w.keep = (sess, buf, x, rl, sgl, y)
+    return w
+
+
+def exl3_head(torch, sz, synth, synth_device, stream, bits):
+    """The lm_head of an EXL3 checkpoint: 151936 x 2048 at `bits` bits a weight for a verify batch, arg-max fused in."""
+    w = Workload()
+    sess = sz.Session(HIDDEN, FF, 8, 2, 0, VOCAB, 8)
+    blob = synth_device.exl3_matrix(torch, 21, HIDDEN, VOCAB, bits)
+    sess.set_head(sz.EXL3(bits), blob.data_ptr())
+    g = torch.Generator(device="cuda")
+    g.manual_seed(14)
+    u = torch.randn((ROWS, HIDDEN), device="cuda", generator=g)
+    ids = torch.zeros(8, dtype=torch.int32, device="cuda")
+    w.step = lambda: sess.head_argmax(ROWS, u.data_ptr(), ids.data_ptr(), stream.handle)
+    w.step_bytes = blob.numel() + ROWS * HIDDEN * 4 + ROWS * 4
+    w.kernel_bytes = {"head_exl3_%d" % bits: blob.numel() + HIDDEN // 128 * 16 * 256}
+    w.dtype = "f32 accumulate over EXL3 f16 codebook weights (f16 matrix cores, inputs as f16 high + low parts)"
+    w.cold_variant = True
+    w.describe = {"workload": "EXL3 lm_head 151936 x 2048 at K = %d for a %d-row verify batch, arg-max fused in (three launches: rotate, "
+                              "product + per-block arg-max, merge)" % (bits, ROWS), "rows": ROWS, "resident_GB": round(blob.numel() / 1e9, 2)}
+    w.counters_key = "exl3head" if (bits == 4 and ROWS == 4) else None
+    w.cpu = ("exl3_matvec", (blob, bits, u[0].cpu().numpy()))
+    w.keep = (sess, blob, u, ids)
     return w
 
 
@@ -295,76 +319,28 @@ def stage_exl3_layer(torch, sz, synth, stream):
     return w
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--layers", type=int, default=48)
-    ap.add_argument("--workload", default="config5", choices=["config1", "config2", "config3", "config4", "config5", "stage", "snapshot"])
-    ap.add_argument("--rows", type=int, default=4, help="rows of the verify batch (config3 and config5; the configurations name 4; 2..8)")
-    ap.add_argument("--tokens", type=int, default=512, help="tokens of the prefill chunk (config4 only; the configuration names 512)")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
-                    help="also launch one plain copy of BYTES bytes, for scaling a profile's memory counters")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs the verify path on ONE GPU (all experts resident in one MI355X's HBM); "
-              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
-        sys.exit(2)
 
-    global ROWS
-    if not 2 <= args.rows <= 8:
-        print("bench.py: --rows takes 2..8", file=sys.stderr)
-        sys.exit(2)
-    ROWS = args.rows
-
-    import torch
-
-    import shadow_engine_amd as sz
-    from shadow_engine_amd import synth, synth_device
-
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible", file=sys.stderr)
-        sys.exit(1)
-    sz.init(0)
-    stream = sz.Stream()
-    if args.workload == "config5":
-        w = exl3_round(torch, sz, synth, synth_device, stream, args.layers, synth_device.layer_rates(2026, args.layers), "config 5")
-    elif args.workload == "config3":
-        w = exl3_round(torch, sz, synth, synth_device, stream, 1, [3], "config 3")
-    elif args.workload == "config1":
-        w = q8_matvec(torch, sz, synth, synth_device, stream)
-    elif args.workload == "config2":
-        w = iq3s_decode(torch, sz, synth, synth_device, stream)
-    elif args.workload == "stage":
-        w = stage_exl3_layer(torch, sz, synth, stream)
-    elif args.workload == "snapshot":
-        w = snapshot_states(torch, sz, stream)
-    else:
-        w = iq3s_prefill(torch, sz, synth, synth_device, stream, args.tokens)
-    torch.cuda.synchronize()
-
-    for _ in range(args.warmup):
+def time_steps(w, stream, sz, torch, steps, warmup):
+    """ms per step of `steps` steps after `warmup` untimed ones, events on the launch stream either side of the timed region."""
+    for _ in range(warmup):
         w.step()
     stream.synchronize()
     torch.cuda.synchronize()
     e0, e1 = sz.Event(), sz.Event()
     t0 = time.perf_counter()
     e0.record(stream.handle)
-    for _ in range(args.steps):
+    for _ in range(steps):
         w.step()
     e1.record(stream.handle)
     stream.synchronize()
     torch.cuda.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
-    ms_per_step = max(e1.since(e0), 0.0) / args.steps
-    w.check()
-    gbps = w.step_bytes / (ms_per_step * 1e-3) / 1e9
+    return max(e1.since(e0), 0.0) / steps, wall_ms / steps
 
-    # every kernel of the step, launch by launch, each with a start and a stop event on the launch stream that carry the
-    # dispatch's own begin and end time stamps (eager steps after the timed region, same buffers)
-    reps = max(2, min(args.steps, 5))
+
+def kernel_times(w, stream, sz, reps):
+    """Every kernel of the step, launch by launch, each between a start and a stop event on the launch stream that carry the
+    dispatch's own begin and end time stamps (eager steps, same buffers)."""
     w.set_eager(True)
     sz.ktime_begin("")
     for _ in range(reps):
@@ -381,45 +357,219 @@ def main():
             per_kernel[name]["GBps"] = w.kernel_bytes[name] / (us * 1e-6) / 1e9
         if name in w.kernel_ops:
             per_kernel[name]["int8_TOPs"] = w.kernel_ops[name] / (us * 1e-6) / 1e12
-    known = [k for k in per_kernel if "GBps" in per_kernel[k]]
-    dom = max(known, key=lambda k: per_kernel[k]["avg_us"] * per_kernel[k]["launches_per_step"]) if known else None
-    roofline = None
-    if dom:
-        a = per_kernel[dom]["GBps"]
-        roofline = {"bound": "hbm", "kernel": dom, "achieved": round(a, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                    "frac": round(a / HBM_PEAK_GBPS, 4), "traffic": w.traffic.get(dom),
-                    "avg_launch_us": round(per_kernel[dom]["avg_us"], 2),
-                    "algorithmic_bytes_per_launch": int(per_kernel[dom]["bytes_per_launch"])}
-        if ROWS == 4 and dom in MEASURED_VALU and w.traffic:
-            g = MEASURED_VALU[dom] / (per_kernel[dom]["avg_us"] * 1e-6) / 1e9
-            roofline["vector_alu"] = {"instructions_per_launch": MEASURED_VALU[dom], "achieved": round(g, 1), "peak": VALU_PEAK_GINST,
-                                      "unit": "G wave64 instructions/s", "frac": round(g / VALU_PEAK_GINST, 4)}
-        if "int8_TOPs" in per_kernel[dom]:
-            t = per_kernel[dom]["int8_TOPs"]
-            roofline["mfma"] = {"achieved": round(t, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s", "frac": round(t / INT8_MFMA_PEAK_TOPS, 5)}
+    return per_kernel
 
-    # configs that fit the caches (1, 2, 3: <= 0.4 GB a step against 256 MB of Infinity Cache + 32 MB of L2) also get a
-    # cold number: a 512 MiB -> 512 MiB copy on the same stream before every timed step, median of the single-step times
-    cold = None
-    if w.cold_variant:
-        nwords = (512 << 20) // 16
-        fsrc = torch.empty(nwords * 16, dtype=torch.uint8, device="cuda").fill_(1)
-        fdst = torch.empty(nwords * 16, dtype=torch.uint8, device="cuda")
-        torch.cuda.synchronize()
-        times = []
-        c0, c1 = sz.Event(), sz.Event()
-        for _ in range(15):
-            sz.launch("copy_words16", (8192, 1, 1), (256, 1, 1), 0, stream.handle,
-                      [sz.Arg.ptr(fsrc.data_ptr()), sz.Arg.ptr(fdst.data_ptr()), sz.Arg.u64(nwords)])
-            c0.record(stream.handle)
-            w.step()
-            c1.record(stream.handle)
-            stream.synchronize()
-            times.append(c1.since(c0))
-        med = float(np.median(times))
-        cold = {"median_us": round(med * 1e3, 2), "GBps": round(w.step_bytes / (med * 1e-3) / 1e9, 1), "reps": len(times),
-                "flush": "1 GiB of copy traffic (512 MiB read + 512 MiB written) on the same stream before every step"}
-        del fsrc, fdst
+
+def roofline_of(w, per_kernel, counters, stale):
+    """The dominant kernel (largest total time among those with known algorithmic bytes) against the HBM roof the metric is
+    defined on and, where hardware counters of this very build are on file, against the vector-ALU roof: a SIMD issues one
+    wave64 vector instruction in 4 cycles, at the shader clock the counters' run measured.  `bound` names the roof that
+    the kernel is nearer to."""
+    known = [k for k in per_kernel if "GBps" in per_kernel[k]]
+    if not known:
+        return None
+    dom = max(known, key=lambda k: per_kernel[k]["avg_us"] * per_kernel[k]["launches_per_step"])
+    a = per_kernel[dom]["GBps"]
+    r = {"bound": "hbm", "kernel": dom, "achieved": round(a, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": round(a / HBM_PEAK_GBPS, 4),
+         "traffic": None, "avg_launch_us": round(per_kernel[dom]["avg_us"], 2),
+         "algorithmic_bytes_per_launch": int(per_kernel[dom]["bytes_per_launch"])}
+    key = getattr(w, "counters_key", None)
+    c = counters["workloads"].get(key, {}).get("kernels", {}).get(dom) if (counters and key and dom not in stale) else None
+    if c:
+        r["traffic"] = c.get("traffic_bytes")
+        if c.get("SQ_INSTS_VALU") and c.get("clock_ghz"):
+            peak = SIMDS * c["clock_ghz"] / 4.0                       # G wave64 vector instructions a second
+            g = c["SQ_INSTS_VALU"] / (per_kernel[dom]["avg_us"] * 1e-6) / 1e9
+            r["vector_alu"] = {"instructions_per_launch": int(c["SQ_INSTS_VALU"]), "achieved": round(g, 1), "peak": round(peak, 1),
+                               "unit": "G wave64 instructions/s", "frac": round(g / peak, 4), "clock_ghz": c["clock_ghz"],
+                               "busy_frac_in_counter_run": c.get("valu_busy_frac")}
+            if g / peak > r["frac"]:
+                r["bound"] = "valu"
+        r["counters"] = "profiles/counters.json"
+    else:
+        r["counters"] = stale.get(dom, "none on file for this workload") if key else "none on file for this workload"
+    if "int8_TOPs" in per_kernel[dom]:
+        t = per_kernel[dom]["int8_TOPs"]
+        r["mfma"] = {"achieved": round(t, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s", "frac": round(t / INT8_MFMA_PEAK_TOPS, 5)}
+    return r
+
+
+def cold_run(w, stream, sz, torch, reps=15):
+    """The median single-step time with 1 GiB of copy traffic on the same stream before every step (the workloads that fit
+    the 256 MB Infinity Cache + L2 between steps)."""
+    nwords = (512 << 20) // 16
+    fsrc = torch.empty(nwords * 16, dtype=torch.uint8, device="cuda").fill_(1)
+    fdst = torch.empty(nwords * 16, dtype=torch.uint8, device="cuda")
+    torch.cuda.synchronize()
+    times = []
+    c0, c1 = sz.Event(), sz.Event()
+    for _ in range(reps):
+        sz.launch("copy_words16", (8192, 1, 1), (256, 1, 1), 0, stream.handle,
+                  [sz.Arg.ptr(fsrc.data_ptr()), sz.Arg.ptr(fdst.data_ptr()), sz.Arg.u64(nwords)])
+        c0.record(stream.handle)
+        w.step()
+        c1.record(stream.handle)
+        stream.synchronize()
+        times.append(c1.since(c0))
+    med = float(np.median(times))
+    del fsrc, fdst
+    return {"median_us": round(med * 1e3, 2), "GBps": round(w.step_bytes / (med * 1e-3) / 1e9, 1), "reps": len(times),
+            "flush": "1 GiB of copy traffic (512 MiB read + 512 MiB written) on the same stream before every step"}
+
+
+def best_of(fn, min_reps, budget_s):
+    """Best and mean seconds of fn() over at least min_reps runs after one warm-up run (crates/shadowzero-model/examples/
+    cpu_expert_bench.rs:34-41 reports the best of its repeats), stopping early only when the budget is spent and 3 runs are in."""
+    fn()
+    times = []
+    t_end = time.perf_counter() + budget_s
+    while len(times) < min_reps or (len(times) < 3):
+        t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+        if time.perf_counter() > t_end and len(times) >= 3:
+            break
+    return min(times), sum(times) / len(times), len(times)
+
+
+def cpu_baseline(kind, args, budget_s=8.0):
+    """The CPU oracle (a restatement of the reference's scalar path, forward.rs:205-249 / exl3.rs:528-599 / cpu_expert.rs) on the
+    host's cores, on a bounded sample of the workload: one thread and all hardware threads, best of >= 20 runs after a warm-up
+    where the budget allows.  It is a baseline only."""
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib as O
+    hw = int(O.lib().orc_hardware_threads())
+    if kind == "exl3_token":
+        (buf, stride), kb, rl0, u0, sgl0 = args
+        ty = O.exl3_type(kb)
+        shape = O.expert_shape(ty, ty, HIDDEN, FF)
+        per_expert = shape.gate_bytes + shape.up_bytes + shape.down_bytes
+        ids = np.argsort(-rl0[0].astype(np.float64), kind="stable")[:TOPK]
+        host = {int(e): buf[int(e) * stride:int(e) * stride + per_expert].cpu().numpy() for e in list(ids) + [NE]}
+        experts = [host.get(e, host[int(ids[0])]) for e in range(NE)]      # only the routed ones are read
+        nbytes = (TOPK + 1) * per_expert
+        run = lambda t: O.moe_token(shape, experts, TOPK, rl0[0], u0[0], shape, host[NE], float(sgl0[0]), t)
+        what = "one token through one layer's MoE block (top-10 + shared EXL3 K=%d experts, %d bytes each)" % (kb, per_expert)
+        # exl3.rs:569-578 splits a projection over its 128-output blocks: 4 threads for gate and up (512 outputs), 16 for down
+        used = min(hw, HIDDEN // 128)
+        note = "a projection is split over its 128-output blocks (exl3.rs:569-578): gate and up run on 4 threads, down on %d" % used
+    elif kind == "iq3_s_token":
+        buf, stride, rl0, u0, sgl0 = args
+        shape = O.expert_shape(O.IQ3_S, O.IQ3_S, HIDDEN, FF)
+        per_expert = shape.gate_bytes + shape.up_bytes + shape.down_bytes
+        ids = np.argsort(-rl0[0].astype(np.float64), kind="stable")[:TOPK]
+        host = {int(e): buf[int(e) * stride:int(e) * stride + per_expert].cpu().numpy() for e in list(ids) + [NE]}
+        experts = [host.get(e, host[int(ids[0])]) for e in range(NE)]
+        nbytes = (TOPK + 1) * per_expert
+        run = lambda t: O.moe_token(shape, experts, TOPK, rl0[0], u0[0], shape, host[NE], float(sgl0[0]), t)
+        what = "one token through one layer's MoE block (top-10 + shared IQ3_S experts, %d bytes each)" % per_expert
+        used, note = hw, "rows split over the threads as forward.rs:205-227"
+    elif kind == "q8_0_matvec":
+        mat, x, rows, cols = args
+        nbytes = mat.size
+        run = lambda t: O.matvec(O.Q8_0, cols, rows, mat, x, t)
+        what = "the Q8_0 %d x %d matrix-vector product of the configuration (CpuBackend::matvec, forward.rs:239-249)" % (rows, cols)
+        used, note = hw, "rows split over the threads as forward.rs:205-227"
+    elif kind == "exl3_matvec":
+        blob, bits, u0 = args
+        rows = 128 * 64                                              # a bounded sample: the first 8192 rows of the vocabulary
+        host = blob[:2 * HIDDEN].cpu().numpy()
+        svh = blob[2 * HIDDEN:2 * HIDDEN + 2 * rows].cpu().numpy()
+        tr = blob[2 * HIDDEN + 2 * VOCAB + 4:].view(HIDDEN // 16, VOCAB // 16, 32 * bits)[:, :rows // 16].contiguous().cpu().numpy()
+        sample = np.concatenate([host, svh, np.array([1, 0, 0, 0], np.uint8), tr.reshape(-1)])
+        nbytes = sample.size
+        run = lambda t: O.exl3_matvec(HIDDEN, rows, bits, sample, u0, threads=t)
+        what = "the head's first %d of %d rows for one input (exl3.rs:528-599 matvec_blob)" % (rows, VOCAB)
+        used, note = min(hw, rows // 128), "one thread a 128-output block (exl3.rs:569-578)"
+    elif kind == "iq3_s_int8_pairs":
+        buf, stride, ids, x8 = args
+        shape = O.expert_shape(O.IQ3_S, O.IQ3_S, HIDDEN, FF)
+        per_expert = shape.gate_bytes + shape.up_bytes + shape.down_bytes
+        pairs = [(t, int(e)) for t in range(x8.shape[0]) for e in ids[t][:2]]          # 16 (token, expert) pairs of the chunk
+        host = {e: buf[e * stride:e * stride + per_expert].cpu().numpy() for _, e in pairs}
+        xq = [O.quantize_act(x8[t], 32) for t in range(x8.shape[0])]
+        nbytes = len(pairs) * per_expert
+        run = lambda t: [O.expert_int8(host[e], HIDDEN, FF, xq[tok][0], xq[tok][1]) for tok, e in pairs]
+        what = "%d (token, expert) pairs of the chunk through the int8-activation expert (cpu_expert.rs:243-339), one after the other" % len(pairs)
+        used, note = 1, "the scalar int8 expert of the oracle runs on one thread"
+    else:
+        return None
+    out = {"unit": "GB/s", "kind": "port", "bytes_per_run": int(nbytes)}
+    modes = [("one_thread", 1)] + ([("all_threads", 0)] if used > 1 else [])
+    for label, t in modes:
+        best, mean, n = best_of(lambda: run(t), 20, budget_s / len(modes))
+        out[label] = {"value": round(nbytes / best / 1e9, 3), "best_us": round(best * 1e6, 1), "mean_us": round(mean * 1e6, 1), "runs": n,
+                      "threads": 1 if t == 1 else used}
+    top = out.get("all_threads", out["one_thread"])
+    out["value"], out["cores"] = top["value"], top["threads"]
+    out["sample"] = "%s with the C++ oracle, best of %d runs after a warm-up; %s (%d hardware threads on the box)" % (what, top["runs"], note, hw)
+    return out
+
+
+def build_workload(name, torch, sz, synth, synth_device, stream, args):
+    if name == "config5":
+        return exl3_round(torch, sz, synth, synth_device, stream, args.layers, synth_device.layer_rates(2026, args.layers), "config 5")
+    if name == "config3":
+        return exl3_round(torch, sz, synth, synth_device, stream, 1, [3], "config 3")
+    if name == "config1":
+        return q8_matvec(torch, sz, synth, synth_device, stream)
+    if name == "config2":
+        return iq3s_decode(torch, sz, synth, synth_device, stream)
+    if name == "config4":
+        return iq3s_prefill(torch, sz, synth, synth_device, stream, args.tokens)
+    if name == "exl3head":
+        return exl3_head(torch, sz, synth, synth_device, stream, args.bits)
+    if name == "stage":
+        return stage_exl3_layer(torch, sz, synth, stream)
+    return snapshot_states(torch, sz, stream)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--layers", type=int, default=48)
+    ap.add_argument("--workload", default="config5", choices=["config1", "config2", "config3", "config4", "config5", "exl3head", "stage", "snapshot"])
+    ap.add_argument("--rows", type=int, default=4, help="rows of the verify batch (config3, config5, exl3head; the configurations name 4; 1..8)")
+    ap.add_argument("--tokens", type=int, default=512, help="tokens of the prefill chunk (config4 only; the configuration names 512)")
+    ap.add_argument("--bits", type=int, default=4, help="bits a weight of the EXL3 head (exl3head only)")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-other-configs", action="store_true", help="default workload only: do not time configurations 1-4 after it")
+    ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
+                    help="also launch one plain copy of BYTES bytes, for scaling a profile's memory counters")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs the verify path on ONE GPU (all experts resident in one MI355X's HBM); "
+              "--gpus %d is not supported" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+
+    global ROWS
+    if not 1 <= args.rows <= 8 or (args.rows == 1 and args.workload in ("config3", "config5")):
+        print("bench.py: --rows takes 2..8 (1..8 for exl3head)", file=sys.stderr)
+        sys.exit(2)
+    ROWS = args.rows
+
+    import torch
+
+    import shadow_engine_amd as sz
+    from shadow_engine_amd import synth, synth_device
+
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible", file=sys.stderr)
+        sys.exit(1)
+    sz.init(0)
+    stream = sz.Stream()
+    w = build_workload(args.workload, torch, sz, synth, synth_device, stream, args)
+    torch.cuda.synchronize()
+
+    ms_per_step, wall_ms = time_steps(w, stream, sz, torch, args.steps, args.warmup)
+    w.check()
+    gbps = w.step_bytes / (ms_per_step * 1e-3) / 1e9
+    per_kernel = kernel_times(w, stream, sz, max(2, min(args.steps, 5)))
+    counters, stale = load_counters(sz)
+    roofline = roofline_of(w, per_kernel, counters, stale)
+    cold = cold_run(w, stream, sz, torch) if w.cold_variant else None
 
     if args.copy_calibration:
         nwords = args.copy_calibration // 16
@@ -429,10 +579,35 @@ def main():
         sz.launch("copy_words16", (8192, 1, 1), (256, 1, 1), 0, stream.handle,
                   [sz.Arg.ptr(src.data_ptr()), sz.Arg.ptr(dst.data_ptr()), sz.Arg.u64(nwords)])
         stream.synchronize()
+        del src, dst
 
     cpu = None
-    if not args.no_cpu_baseline and hasattr(w, "cpu_args"):
-        cpu = cpu_baseline(torch, *w.cpu_args)
+    if not args.no_cpu_baseline and hasattr(w, "cpu"):
+        cpu = cpu_baseline(*w.cpu)
+
+    # the other configurations of the path, once each after the timed region of the default one (they are parity-test cases
+    # first): time, algorithmic GB/s against 8 TB/s, warm and cold, their dominant kernel, and the CPU oracle beside each
+    others = None
+    if args.workload == "config5" and args.layers == 48 and ROWS == 4 and not args.no_other_configs:
+        others = {}
+        for name in ("config1", "config2", "config3", "config4"):
+            ow = build_workload(name, torch, sz, synth, synth_device, stream, args)
+            torch.cuda.synchronize()
+            oms, _ = time_steps(ow, stream, sz, torch, 30, 3)
+            ow.check()
+            opk = kernel_times(ow, stream, sz, 3)
+            og = ow.step_bytes / (oms * 1e-3) / 1e9
+            entry = {"workload": ow.describe["workload"], "us_per_step": round(oms * 1e3, 2), "GBps": round(og, 1),
+                     "frac_of_8TBps": round(og / HBM_PEAK_GBPS, 4), "algorithmic_bytes_per_step": int(ow.step_bytes),
+                     "roofline": roofline_of(ow, opk, counters, stale),
+                     "cold_cache": cold_run(ow, stream, sz, torch, 9) if ow.cold_variant else None}
+            if name == "config2":
+                entry["us_per_layer"] = round(oms * 1e3 / ow.describe["layers"], 2)
+            if not args.no_cpu_baseline and hasattr(ow, "cpu"):
+                entry["cpu_baseline"] = cpu_baseline(*ow.cpu, budget_s=2.0)
+            others[name] = entry
+            del ow
+            torch.cuda.empty_cache()
 
     line = {
         "metric": "MoE quant-matvec HBM GB/s (% of 8 TB/s); K=3 spec-verify round µs",
@@ -440,41 +615,14 @@ def main():
         "ms_per_step": round(ms_per_step, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": w.dtype, "data": "synthetic", "config": w.describe,
         "round_us": round(ms_per_step * 1e3, 1), "pct_of_8TBps": round(100 * gbps / HBM_PEAK_GBPS, 2),
-        "algorithmic_bytes_per_step": int(w.step_bytes), "host_wall_ms_per_step": round(wall_ms / args.steps, 4),
+        "algorithmic_bytes_per_step": int(w.step_bytes), "host_wall_ms_per_step": round(wall_ms, 4),
         "roofline": roofline, "kernels": {k: {kk: (round(vv, 2) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in per_kernel.items()},
         "cpu_baseline": cpu, "cold_cache": cold,
     }
+    if others is not None:
+        line["other_configs"] = others
     line.update(w.extra)
     print(json.dumps(line))
-
-
-def cpu_baseline(torch, layer0, kb, rl0, u0, sgl0):
-    """The CPU oracle (a restatement of the reference's scalar path) on the host's cores: whole MoE tokens of layer 0,
-    repeated until about 10 s of work, reported as expert-weight GB/s."""
-    sys.path.insert(0, os.path.join(ROOT, "tests"))
-    import oracle_lib as O
-    buf, stride = layer0
-    ty = O.exl3_type(kb)
-    shape = O.expert_shape(ty, ty, HIDDEN, FF)
-    per_expert = shape.gate_bytes + shape.up_bytes + shape.down_bytes
-    ids = np.argsort(-rl0[0].astype(np.float64), kind="stable")[:TOPK]
-    host = {}
-    for e in list(ids) + [NE]:
-        host[int(e)] = buf[int(e) * stride:int(e) * stride + per_expert].cpu().numpy()
-    experts = [host.get(e, host[int(ids[0])]) for e in range(NE)]      # only the routed ones are read
-    threads = O.lib().orc_hardware_threads()
-    t0 = time.perf_counter()
-    reps = 0
-    while True:
-        O.moe_token(shape, experts, TOPK, rl0[0], u0[0], shape, host[NE], float(sgl0[0]), threads)
-        reps += 1
-        dt = time.perf_counter() - t0
-        if dt > 10.0 or reps >= 2000:
-            break
-    nbytes = reps * (TOPK + 1) * per_expert
-    return {"value": round(nbytes / dt / 1e9, 3), "unit": "GB/s", "cores": int(threads), "kind": "port",
-            "sample": "%d x one token through layer 0's MoE block (top-10 + shared EXL3 K=%d experts, %d bytes each) in %.1f s with the "
-                      "C++ oracle, rows/blocks split over all hardware threads as forward.rs:205-227" % (reps, kb, per_expert, dt)}
 
 
 if __name__ == "__main__":

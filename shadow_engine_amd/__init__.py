@@ -453,6 +453,18 @@ def matvec_cols_static(ggml_type, w_dev, cols, rows, x_dev, xs, y_dev, ys, m, st
     check(lib().sz_matvec_cols_static(ggml_type, w_dev, cols, rows, x_dev, xs, y_dev, ys, m, stream))
 
 
+def program_keys():
+    """{kernel file: cache key of the code object built ahead of time from its current source}."""
+    out = {}
+    L = lib()
+    for i in range(L.sz_program_file_count()):
+        name = L.sz_program_file_name(i)
+        key = C.create_string_buffer(65)
+        if L.sz_program_cache_key(name, key) == 0:
+            out[name.decode()] = key.value.decode()
+    return out
+
+
 def verify_accept(ids, drafts):
     """engine.rs:2377-2408: keep = 1 + the leading drafts that equal the model's choices."""
     ids = np.ascontiguousarray(ids, np.uint32)

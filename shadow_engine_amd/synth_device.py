@@ -30,6 +30,22 @@ def exl3_layer(torch, seed, hidden, ff, ne, bits):
     return buf.reshape(-1), stride
 
 
+def exl3_matrix(torch, seed, inf, outf, bits):
+    """uint8[exl3_blob_len]: one EXL3 projection (the lm_head's shape when outf is the vocabulary): random trellis words,
+    suh = +-1, svh = 0.3 + U[0,1)."""
+    g = torch.Generator(device="cuda")
+    g.manual_seed(seed)
+    n = synth.exl3_blob_len(inf, outf, bits)
+    buf = torch.randint(0, 256, (n,), dtype=torch.uint8, device="cuda", generator=g)
+    sign = torch.randint(0, 2, (inf,), device="cuda", generator=g)
+    suh = torch.where(sign == 0, 0x3C00, 0xBC00).to(torch.int16)
+    svh = (0.3 + torch.randint(0, 100, (outf,), device="cuda", generator=g).float() / 100.0).half()
+    buf[:2 * inf] = suh.view(torch.uint8)
+    buf[2 * inf:2 * inf + 2 * outf] = svh.view(torch.uint8)
+    buf[2 * inf + 2 * outf:2 * inf + 2 * outf + 4] = torch.tensor([1, 0, 0, 0], dtype=torch.uint8, device="cuda")
+    return buf
+
+
 def q8_0_head(torch, seed, vocab, hidden):
     """uint8[vocab * hidden / 32 * 34]: the head as Q8_0 rows."""
     g = torch.Generator(device="cuda")
