@@ -184,7 +184,9 @@ def iq3s_decode(torch, sz, synth, synth_device, stream, L=8):
     w.step = step
     w.step_bytes = L * ((TOPK + 1) * expert + (2 * HIDDEN + NE + 1) * 4)
     gu, _, dn = synth.expert_bytes(sz.IQ3_S, HIDDEN, FF)
-    w.kernel_bytes = {"verify_gate_up_iq3_s": (TOPK + 1) * 2 * gu + (HIDDEN + NE) * 4 + (TOPK + 1) * 2 * FF * 4,
+    w.kernel_bytes = {"decode_gate_up_iq3_s": (TOPK + 1) * 2 * gu + (HIDDEN + NE) * 4 + (TOPK + 1) * FF * 4,      # one token: two launches
+                      "decode_down_combine_iq3_s": (TOPK + 1) * dn + (TOPK + 1) * FF * 4 + HIDDEN * 4,
+                      "verify_gate_up_iq3_s": (TOPK + 1) * 2 * gu + (HIDDEN + NE) * 4 + (TOPK + 1) * 2 * FF * 4,   # the three-launch form
                       "verify_down_iq3_s": (TOPK + 1) * dn + (TOPK + 1) * (2 * FF + HIDDEN) * 4,
                       "matvec_grouped_iq3_s": (TOPK + 1) * expert / 2.0}      # the planned form: gate+up in one launch, down in the other: the mean
     w.dtype = "f32 accumulate over IQ3_S grid weights"
@@ -392,6 +394,32 @@ def roofline_of(w, per_kernel, counters, stale):
         t = per_kernel[dom]["int8_TOPs"]
         r["mfma"] = {"achieved": round(t, 2), "peak": INT8_MFMA_PEAK_TOPS, "unit": "TOP/s", "frac": round(t / INT8_MFMA_PEAK_TOPS, 5)}
     return r
+
+
+def vector_floor(w, per_kernel, counters, stale, ms_per_step):
+    """The time a step's counted vector instructions would take if every one of the 1024 SIMDs issued one every 4 cycles for
+    the whole step (no launch boundaries, no waits, perfectly even work): a floor for this instruction count, from the
+    counters on file; None unless every kernel of the step that has algorithmic bytes has current counters."""
+    key = getattr(w, "counters_key", None)
+    ks = counters["workloads"].get(key, {}).get("kernels", {}) if (counters and key) else {}
+    cycles, clocks, n = 0.0, [], 0
+    for name, v in per_kernel.items():
+        c = ks.get(name)
+        if name in stale or not c or not c.get("SQ_INSTS_VALU"):
+            if "bytes_per_launch" in v:
+                return None
+            continue
+        cycles += c["SQ_INSTS_VALU"] * v["launches_per_step"] * 4.0 / SIMDS
+        n += c["SQ_INSTS_VALU"] * v["launches_per_step"]
+        if c.get("clock_ghz", 0) > 1.0:
+            clocks.append(c["clock_ghz"])
+    if not clocks:
+        return None
+    ghz = sum(clocks) / len(clocks)
+    us = cycles / ghz / 1e3
+    return {"us_per_step": round(us, 1), "frac_of_measured_step": round(us / (ms_per_step * 1e3), 4), "vector_instructions_per_step": int(n),
+            "clock_ghz": round(ghz, 3), "means": "counted wave64 vector instructions of a step x 4 cycles / 1024 SIMDs / clock: the step cannot be "
+            "shorter than this without issuing fewer instructions"}
 
 
 def cold_run(w, stream, sz, torch, reps=15):
@@ -616,7 +644,7 @@ def main():
         "dtype": w.dtype, "data": "synthetic", "config": w.describe,
         "round_us": round(ms_per_step * 1e3, 1), "pct_of_8TBps": round(100 * gbps / HBM_PEAK_GBPS, 2),
         "algorithmic_bytes_per_step": int(w.step_bytes), "host_wall_ms_per_step": round(wall_ms, 4),
-        "roofline": roofline, "kernels": {k: {kk: (round(vv, 2) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in per_kernel.items()},
+        "roofline": roofline, "vector_alu_floor": vector_floor(w, per_kernel, counters, stale, ms_per_step), "kernels": {k: {kk: (round(vv, 2) if isinstance(vv, float) else vv) for kk, vv in v.items()} for k, v in per_kernel.items()},
         "cpu_baseline": cpu, "cold_cache": cold,
     }
     if others is not None:

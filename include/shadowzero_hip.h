@@ -212,7 +212,8 @@ int32_t sz_copy_ranges(const uint64_t* ranges, uint32_t n, uint64_t stream);
 
 /* The session's batch buffers, for tests and measurements (device addresses; the contents are those of the last call):
  * 0 the plan (chosen experts u32[m][k], weights f32[m][k], counts u32[m] for the fused layers), 1 the split-k partial sums of
- * gate and up, 2 the down products.  0 for any other `which`. */
+ * gate and up, 2 the down products (EXL3 layers); 3 the gate and up rows, 4 the down rows of a GGUF layer's pairs.  0 for any other
+ * `which`. */
 uint64_t sz_session_buffer(sz_session*, int32_t which);
 
 /* A whole verify round over device-resident inputs: for every layer l the MoE block on u[l][m][hidden] with rl[l][m][ne]

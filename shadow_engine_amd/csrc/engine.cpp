@@ -375,6 +375,27 @@ int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, ui
         const uint64_t part = matrix_bytes(f, c.hidden, c.ff);
         if (part >> 32) return fail("sz_moe_layer_verify: a projection of 4 GiB or more");
         const uint32_t rb_gu = c.hidden / f.qk * f.bb, rb_d = c.ff / f.qk * f.bb;
+        // One token: two launches.  Launch 1 hands over act = silu(gate) * up and the routing weights, launch 2 owns a row chunk
+        // for all of the token's experts and adds them up itself (SHADOWZERO_GGUF_THREE_LAUNCH=1 keeps the general form).
+        const bool three = std::getenv("SHADOWZERO_GGUF_THREE_LAUNCH") != nullptr;
+        const uint32_t uh = c.hidden / 32, uf = c.ff / 32;
+        if (m == 1 && !three && c.hidden % 32 == 0 && c.ff % 32 == 0 && uh <= 64 && 64 % uh == 0 && uf <= 64 && 64 % uf == 0 && c.top_k <= 16) {
+            const uint32_t rp = 8, rd = std::max(4u, 64 / uf);
+            const uint32_t rs_gu = (rp * rb_gu + 31) / 16 * 16, rs_d = (rd * rb_d + 31) / 16 * 16;
+            const uint32_t Sd = c.top_k + (shared ? 1 : 0);
+            if (c.ff % rp == 0 && c.hidden % rd == 0 && 2 * rs_gu <= 16384 && Sd * rs_d <= 16384 && Sd * c.ff <= 8192) {
+                const std::string d1 = "decode_gate_up_" + tag, d2 = "decode_down_combine_" + tag;
+                {
+                    const sz_arg a[] = {P(rl), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(u), P(plan), P(s->eg.ptr),
+                                        U32(c.n_expert), U32(c.top_k), U32(m), U32(c.hidden), U32(c.ff), U32(rp)};
+                    if (launch(d1.c_str(), c.ff / rp, S, 1, 512, 2 * rs_gu, stream, a)) return 1;   // 8 waves: a gate row and an up row each at hidden 2048
+                }
+                s->last_fused = true;
+                const sz_arg a[] = {U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(plan), P(s->eg.ptr), P(sgl), P(y),
+                                    U32(c.top_k), U32(c.hidden), U32(c.ff), U32(rd)};
+                return launch(d2.c_str(), c.hidden / rd, 1, 1, 64 * std::min(16u, std::max(4u, Sd)), Sd * rs_d + Sd * uf * 144, stream, a);   // a wave a pair
+            }
+        }
         const std::string k1 = "verify_gate_up_" + tag, k2 = "verify_down_" + tag;
         {
             const sz_arg a[] = {P(rl), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(u), P(plan), P(s->eg.ptr),
@@ -644,7 +665,7 @@ int32_t sz_session_set_head(sz_session* s, int32_t ty, uint64_t w) {
 
 uint64_t sz_session_buffer(sz_session* s, int32_t which) {
     if (!s) return 0;
-    return which == 0 ? s->plan.ptr : which == 1 ? s->part.ptr : which == 2 ? s->dn.ptr : 0;
+    return which == 0 ? s->plan.ptr : which == 1 ? s->part.ptr : which == 2 ? s->dn.ptr : which == 3 ? s->eg.ptr : which == 4 ? s->eo.ptr : 0;
 }
 
 int32_t sz_session_set_graph(sz_session* s, int32_t enabled) {

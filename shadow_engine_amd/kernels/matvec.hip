@@ -500,7 +500,9 @@ __device__ __forceinline__ void verify_gate_up_gguf(const float* logits, u64 eba
     if (pair < G) {
         const u32 t = pair % k;
         if (wave == ((blockIdx.x + blockIdx.y) & 3u)) {
+            __builtin_amdgcn_s_setprio(3);   // every other wave of the workgroup waits for this one
             route_id_of_rank(logits + (u64) j * ne, ne, k, t, lane, s_ex, s_top);   // only s_top[t] is read
+            __builtin_amdgcn_s_setprio(0);
             if (sel == 0 && blockIdx.x == 0 && lane == 0) ((u32*) pbuf)[pair] = s_top[t];
         }
         __syncthreads();
@@ -581,6 +583,283 @@ __device__ __forceinline__ void verify_down_gguf(const float* logits, u64 ebase,
     for (u32 i = threadIdx.x; i < ff; i += 256) act[i] = siluf_ref(g[i]) * up[i];
     __syncthreads();
     rows_body<F, 1>(w, hidden, ff, rpb, xp, yp, nullptr, NoAfter());
+}
+
+// ------------------------------------------------------------------------ the decode layer (one token) in two launches
+// For a single token the down launch can own a row chunk for ALL of the token's experts, weight and add them in rank order
+// itself, and the combine launch goes away.  Launch 1 then hands over act = silu(gate) * up instead of the two sums (a
+// workgroup takes the same rows of gate and of up), and one wave of it computes the routing weights, which launch 2 only reads.
+// pbuf as above; act holds S rows of ff floats.  The sums are rows_body's single-input sums and the combine is
+// moe_combine_qwen_rows's arithmetic, so y has the bits of the three-launch form.
+
+// The same weights without the sum over all experts: w_t = ex_t / (sum of the chosen ex), which is what the reference's
+// (ex_t / z) / (sum of the chosen ex / z) is before rounding; in f64 the two differ by a few units in the last place at
+// most, far below the f32 the weights are rounded to.  Ten exponentials instead of ne: for a caller with the chosen
+// experts in LDS and a wave to spare but no time.  Lane t < k returns the weight of rank t; *count as route_weights.
+__device__ __forceinline__ float route_weights_chosen(const float* lg, u32 ne, u32 k, u32 lane, const u32* top, u32* count) {
+    float lv[8];
+#pragma unroll
+    for (int q = 0; q < 8; q++) lv[q] = lg[min(q * 64 + lane, ne - 1)];
+    const u32 e = lane < k ? top[lane] : 0xffffffffu;
+    const float le = lg[e != 0xffffffffu ? e : 0];
+    float mx = -3.402823466e+38f;
+#pragma unroll
+    for (int q = 0; q < 8; q++)
+        if (q * 64 + lane < ne) mx = fmaxf(mx, lv[q]);
+    mx = wave_max_f32(mx);
+    const double mine = e != 0xffffffffu ? exp((double) (le - mx)) : 0.0;
+    double tz = 0.0;
+    u32 kk = 0;
+#pragma unroll 1
+    for (u32 t = 0; t < k; t++) {
+        const double v = __shfl(mine, t, SZ_WAVE);
+        if (__shfl(e, t, SZ_WAVE) != 0xffffffffu) {
+            tz += v;
+            kk++;
+        }
+    }
+    *count = kk;
+    return e != 0xffffffffu ? (float) (mine / tz) : 0.0f;
+}
+
+// Copies `n` spans of `span` bytes into LDS regions of `rs` bytes each (a multiple of 16, at least span + 15): span p starts
+// at global address g0(p) and lands so that its first byte is at byte (g0(p) & 15) of region p, which starts at dynamic LDS
+// byte p * rs; a null g0(p) skips the span.  All the loads of a thread (at most 4: n * rs / 16 <= 1024) are in flight
+// before its first store; a chunk that reaches outside its span is read byte by byte, so nothing outside the spans is touched.
+template <class Addr>
+__device__ __forceinline__ void stage_spans(Addr g0, u32 n, u32 span, u32 rs, u32 tid) {
+    const u32 ch = rs / 16, total = n * ch, nthr = blockDim.x;
+    u32x4 v[4];
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const u32 i = tid + nthr * r;
+        v[r] = u32x4{0, 0, 0, 0};
+        if (i < total) {
+            const u32 p = i / ch, c = i % ch;
+            const u8* g = g0(p);
+            if (g) {
+                const u32 head = (u32) ((u64) g & 15);
+                const u8* a0 = g - head;
+                const u32 lo = c * 16, end = head + span;
+                if (lo >= head && lo + 16 <= end) {
+                    v[r] = *(const u32x4*) (a0 + lo);
+                } else if (lo < end && lo + 16 > head) {
+                    u32 w[4] = {0, 0, 0, 0};
+                    for (u32 b = 0; b < 16; b++) {
+                        const u32 idx = lo + b;
+                        if (idx >= head && idx < end) w[b / 4] |= (u32) a0[idx] << (8 * (b % 4));
+                    }
+                    v[r] = u32x4{w[0], w[1], w[2], w[3]};
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; r++) {
+        const u32 i = tid + nthr * r;
+        if (i < total) ((u32x4*) sz_dyn_lds)[i] = v[r];
+    }
+}
+
+// Launch 1: as verify_gate_up_gguf for one chunk a workgroup, but the workgroup takes rows [rp blockIdx.x, +rp) of gate AND
+// of up and writes act.  The workgroup blockIdx.x == 0 of every token's last pair (the shared expert's, or rank 0's when
+// there is none) also selects all k experts on a wave of its own and leaves ids, weights and count in pbuf.
+// grid = (ff / rp, S), block 256 to 1024 (a wave takes the rows wave, wave + waves, ..), dynamic LDS = 2 * (rp * row bytes + 32); hidden / 32 divides 64, rp divides ff.
+template <class F>
+__device__ __forceinline__ void decode_gate_up_gguf(const float* logits, u64 ebase, u64 estride, u64 shbase, u32 part, const float* u, u8* pbuf,
+                                                    float* act, u32 ne, u32 k, u32 m, u32 hidden, u32 ff, u32 rp) {
+    __shared__ u32 s_top[16], s_all[16];
+    __shared__ double s_ex[512], s_ex_all[512];   // only the exact fallback of the routing touches them
+    __shared__ __attribute__((aligned(16))) float s_x[64 * XU_PITCH];
+    const u32 G = m * k, S = G + m;
+    const u32 wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const u32 pair = blockIdx.y;
+    const u32 j = pair < G ? pair / k : pair - G;
+    if (pair >= G && !shbase) return;
+    for (u32 i = threadIdx.x; i < hidden / 4; i += blockDim.x) *(f32x4*) (s_x + (i / 8) * XU_PITCH + (i % 8) * 4) = ((const f32x4*) (u + (u64) j * hidden))[i];
+    if constexpr (F::BB == 110) {
+        for (u32 i = threadIdx.x; i < 512; i += blockDim.x) sz_iq3s_grid[i] = IQ3S_GRID[i];
+    }
+    const u32 rwave = (blockIdx.x + blockIdx.y) & 3u;             // the wave that finds this pair's expert
+    const bool all = blockIdx.x == 0 && pair == (shbase ? G + j : j * k);
+    if (all && wave == ((rwave + 1) & 3u)) {
+        const float* lg = logits + (u64) j * ne;
+        __builtin_amdgcn_s_setprio(3);
+        route_ids(lg, ne, k, lane, s_ex_all, s_all);
+        u32 kk;
+        const float wt = route_weights_chosen(lg, ne, k, lane, s_all, &kk);
+        if (lane < k) {
+            ((u32*) pbuf)[j * k + lane] = s_all[lane];
+            ((float*) (pbuf + G * 4))[j * k + lane] = wt;
+        }
+        if (lane == 0) ((u32*) (pbuf + 2 * G * 4))[j] = kk;
+        __builtin_amdgcn_s_setprio(0);
+    }
+    const u8* w;
+    if (pair < G) {
+        const u32 t = pair % k;
+        if (wave == rwave) {
+            // the wave every other wave of the workgroup waits for: it goes first where it shares a SIMD with waves of
+            // workgroups that are already multiplying
+            __builtin_amdgcn_s_setprio(3);
+            route_id_of_rank(logits + (u64) j * ne, ne, k, t, lane, s_ex, s_top);   // only s_top[t] is read
+            __builtin_amdgcn_s_setprio(0);
+        }
+        __syncthreads();
+        const u32 e = s_top[t];
+        if (e == 0xffffffffu) return;
+        w = (const u8*) (ebase + e * estride);
+    } else {
+        w = (const u8*) shbase;
+    }
+    const u32 rb = hidden / F::QK * F::BB, r0 = blockIdx.x * rp;
+    const u32 rs = (rp * rb + 31) / 16 * 16;
+    stage_spans([&](u32 p) { return w + (u64) p * part + (u64) r0 * rb; }, 2, rp * rb, rs, threadIdx.x);
+    __syncthreads();       // the rows, and for the shared expert's pairs also s_x and the table
+    const u32 hg = (u32) ((u64) (w + (u64) r0 * rb) & 15), hu = rs + (u32) ((u64) (w + (u64) part + (u64) r0 * rb) & 15);
+    const u32 U = hidden / 32, RG = 64 / U, sub = lane / U, ul = lane % U;
+    float x[32][1];
+    unit_from_lds(s_x, ul, x);
+    float* o = act + (u64) pair * ff + r0;
+    for (u32 lr = wave * RG + sub; lr < rp; lr += (blockDim.x / 64) * RG) {
+        float g[1] = {0.0f}, up[1] = {0.0f};
+        unit_dot<F, 1>(hg + lr * rb, ul, x, g);
+        unit_dot<F, 1>(hu + lr * rb, ul, x, up);
+        g[0] = seg_sum_rt(g[0], U, lane);
+        up[0] = seg_sum_rt(up[0], U, lane);
+        if (ul == 0) o[lr] = siluf_ref(g[0]) * up[0];
+    }
+}
+
+// Launch 2 for one token: rows [rd blockIdx.x, +rd) of the down matrix of every chosen expert and of the shared one against
+// that pair's act, then y = the sum in rank order of weight * row, plus sigmoid(gate logit) * the shared expert's row.
+// grid = hidden / rd, block 256 to 1024 (a wave takes the pairs wave, wave + waves, ..), dynamic LDS = S * region + S * (ff / 32) * 144 with region = rd * row bytes + 31 rounded
+// down to 16; ff / 32 divides 64, 64 / (ff / 32) divides rd, rd divides hidden, S * region <= 16 KiB, S * ff <= 8192, k <= 16.
+template <class F>
+__device__ __forceinline__ void decode_down_combine_gguf(u64 ebase, u64 estride, u64 shbase, u32 part, const u8* pbuf, const float* act,
+                                                         const float* gl, float* y, u32 k, u32 hidden, u32 ff, u32 rd) {
+    __shared__ float s_eo[17][64];
+    __shared__ float s_w[16];
+    const u32 G = k, S = shbase ? k + 1 : k;
+    const u32 tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const u32 rb = ff / F::QK * F::BB, r0 = blockIdx.x * rd;
+    const u32 rs = (rd * rb + 31) / 16 * 16;
+    const u32 U = ff / 32, nthr = blockDim.x;
+    float* s_act = (float*) ((u8*) sz_dyn_lds + S * rs);
+    // every load goes out before anything is waited for: the pairs' act, the chosen ids, then the rows
+    const u32 n4 = ff / 4, pieces = S * n4;
+    f32x4 av[8];
+#pragma unroll
+    for (int h = 0; h < 8; h++) av[h] = ((const f32x4*) act)[min(tid + nthr * h, pieces - 1)];
+    const u32 myid = ((const u32*) pbuf)[min(lane, k - 1)];
+    const float wt = ((const float*) (pbuf + G * 4))[min(lane, k - 1)];
+    const u32 cnt = ((const u32*) (pbuf + 2 * G * 4))[0];
+    const float glv = shbase ? gl[0] : 0.0f;
+    if constexpr (F::BB == 110) {
+        for (u32 i = tid; i < 512; i += nthr) sz_iq3s_grid[i] = IQ3S_GRID[i];
+    }
+    if (wave == 0 && lane < 16) s_w[lane] = lane < k ? wt : 0.0f;
+    // the experts' addresses need the ids, which every wave holds in its lanes 0..k-1: a wave-level broadcast
+    auto row_of = [&](u32 p) -> const u8* {
+        if (p >= G) return (const u8*) (shbase + 2 * (u64) part + (u64) r0 * rb);
+        const u32 e = (u32) __shfl((int) myid, (int) p, SZ_WAVE);
+        return e == 0xffffffffu ? nullptr : (const u8*) (ebase + e * estride + 2 * (u64) part + (u64) r0 * rb);
+    };
+    // as stage_spans, with every lane fetching the id of its chunk's pair from the lane that holds it
+    {
+        const u32 ch = rs / 16, total = S * ch;
+        u32x4 v[4];
+        const u8* src[4];
+        u32 lo[4], hd[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const u32 i = min(tid + nthr * r, total - 1), p = i / ch;
+            const u8* g = nullptr;
+            // (p differs between the lanes of a wave: every lane fetches its pair's id from the lane that holds it)
+            if (p >= G) g = (const u8*) (shbase + 2 * (u64) part + (u64) r0 * rb);
+            const u32 e = (u32) __shfl((int) myid, (int) min(p, k - 1), SZ_WAVE);
+            if (p < G && e != 0xffffffffu) g = (const u8*) (ebase + e * estride + 2 * (u64) part + (u64) r0 * rb);
+            src[r] = g;
+            hd[r] = (u32) ((u64) g & 15);
+            lo[r] = (i % ch) * 16;
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            v[r] = u32x4{0, 0, 0, 0};
+            const u32 i = tid + nthr * r;
+            if (i < total && src[r]) {
+                const u8* a0 = src[r] - hd[r];
+                const u32 end = hd[r] + rd * rb;
+                if (lo[r] >= hd[r] && lo[r] + 16 <= end) {
+                    v[r] = *(const u32x4*) (a0 + lo[r]);
+                } else if (lo[r] < end && lo[r] + 16 > hd[r]) {
+                    u32 w[4] = {0, 0, 0, 0};
+                    for (u32 b = 0; b < 16; b++) {
+                        const u32 idx = lo[r] + b;
+                        if (idx >= hd[r] && idx < end) w[b / 4] |= (u32) a0[idx] << (8 * (b % 4));
+                    }
+                    v[r] = u32x4{w[0], w[1], w[2], w[3]};
+                }
+            }
+        }
+#pragma unroll
+        for (int h = 0; h < 8; h++) {
+            const u32 i = tid + nthr * h;
+            if (i < pieces) {
+                const u32 p = i / n4, q = i % n4;
+                *(f32x4*) (s_act + (p * U + q / 8) * XU_PITCH + (q % 8) * 4) = av[h];
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < 4; r++) {
+            const u32 i = tid + nthr * r;
+            if (i < total) ((u32x4*) sz_dyn_lds)[i] = v[r];
+        }
+    }
+    __syncthreads();
+    const u32 RG = 64 / U, sub = lane / U, ul = lane % U;
+    for (u32 p = wave; p < S; p += nthr / 64) {
+        const u8* g = row_of(p);
+        if (!g) continue;                       // a masked rank: nothing was staged and nothing is added
+        const u32 head = p * rs + (u32) ((u64) g & 15);
+        float x[32][1];
+        unit_from_lds(s_act + p * U * XU_PITCH, ul, x);
+        for (u32 lr = sub; lr < rd; lr += RG) {
+            float tot[1] = {0.0f};
+            unit_dot<F, 1>(head + lr * rb, ul, x, tot);
+            tot[0] = seg_sum_rt(tot[0], U, lane);
+            if (ul == 0) s_eo[p][lr] = tot[0];
+        }
+    }
+    __syncthreads();
+    if (tid < rd) {
+        float acc = 0.0f;
+        for (u32 t = 0; t < k; t++)
+            if (t < cnt) acc += s_w[t] * s_eo[t][tid];
+        if (shbase) acc += sigmoidf_ref(glv) * s_eo[G][tid];
+        y[r0 + tid] = acc;
+    }
+}
+
+extern "C" __global__ void __launch_bounds__(1024) decode_gate_up_q8_0(const float* logits, u64 ebase, u64 estride, u64 shbase, u32 part,
+                                                                      const float* u, u8* pbuf, float* act, u32 ne, u32 k, u32 m, u32 hidden,
+                                                                      u32 ff, u32 rp) {
+    decode_gate_up_gguf<Q80>(logits, ebase, estride, shbase, part, u, pbuf, act, ne, k, m, hidden, ff, rp);
+}
+extern "C" __global__ void __launch_bounds__(1024) decode_gate_up_iq3_s(const float* logits, u64 ebase, u64 estride, u64 shbase, u32 part,
+                                                                       const float* u, u8* pbuf, float* act, u32 ne, u32 k, u32 m, u32 hidden,
+                                                                       u32 ff, u32 rp) {
+    decode_gate_up_gguf<IQ3S>(logits, ebase, estride, shbase, part, u, pbuf, act, ne, k, m, hidden, ff, rp);
+}
+extern "C" __global__ void __launch_bounds__(1024) decode_down_combine_q8_0(u64 ebase, u64 estride, u64 shbase, u32 part, const u8* pbuf,
+                                                                           const float* act, const float* gl, float* y, u32 k, u32 hidden,
+                                                                           u32 ff, u32 rd) {
+    decode_down_combine_gguf<Q80>(ebase, estride, shbase, part, pbuf, act, gl, y, k, hidden, ff, rd);
+}
+extern "C" __global__ void __launch_bounds__(1024) decode_down_combine_iq3_s(u64 ebase, u64 estride, u64 shbase, u32 part, const u8* pbuf,
+                                                                            const float* act, const float* gl, float* y, u32 k, u32 hidden,
+                                                                            u32 ff, u32 rd) {
+    decode_down_combine_gguf<IQ3S>(ebase, estride, shbase, part, pbuf, act, gl, y, k, hidden, ff, rd);
 }
 
 extern "C" __global__ void __launch_bounds__(256) verify_gate_up_q8_0(const float* logits, u64 ebase, u64 estride, u64 shbase, u32 part,

@@ -344,6 +344,53 @@ def test_moe_layer_verify_planned_form_matches_the_oracle(gpu, monkeypatch, ty, 
     run_moe_layer_case(gpu, ty, hidden, ff, ne, k, m, shared)
 
 
+@pytest.mark.parametrize("ty,hidden,ff,ne,k,shared", [
+    (sz.IQ3_S, 2048, 512, 96, 10, True),           # the decode shape
+    (sz.IQ3_S, 1024, 256, 24, 16, True),           # k = 16, the most the session takes; 8 units a down row
+    (sz.IQ3_S, 512, 1024, 8, 3, True),             # 32 units a down row
+    (sz.IQ3_S, 512, 256, 8, 3, False),             # no shared expert: rank 0's workgroup computes the weights; 8 units a down row
+    (sz.Q8_0, 1024, 512, 12, 4, True),
+    (sz.Q8_0, 512, 256, 16, 4, False),
+    (sz.Q8_0, 2048, 2048, 6, 2, True),             # too large for launch 2's staging: the call falls back to three launches
+])
+def test_one_token_layer_in_two_launches(gpu, monkeypatch, ty, hidden, ff, ne, k, shared):
+    """A single token takes the two-launch form (act and the routing weights out of launch 1, the down rows of all experts and
+    the rank-order sum in launch 2): against the oracle, with masked experts (fewer finite logits than k, and none but one),
+    and against the three-launch form of the same call (the same sums; the weights may differ in the last bit, launch 1 sums
+    only the chosen experts' exponentials)."""
+    rng = np.random.default_rng(ty * 7 + hidden + k)
+    dbuf, stride, blobs, sh = build_layer(gpu, rng, ty, hidden, ff, ne, shared)
+    s = sz.Session(hidden, ff, ne, k, 1, 0, 8)
+    s.set_layer(0, ty, dbuf.data_ptr(), stride, ty if shared else 0, dbuf.data_ptr() + ne * stride if shared else 0)
+    for finite in (ne, max(1, k - 1), 1):
+        u = rng.normal(size=(1, hidden)).astype(np.float32)
+        logits = rng.normal(size=(1, ne)).astype(np.float32)
+        if finite < ne:
+            row = np.full(ne, -np.inf, np.float32)
+            keep = rng.choice(ne, finite, replace=False)
+            row[keep] = logits[0, keep]
+            logits[0] = row
+        sgl = rng.normal(size=1).astype(np.float32)
+        du, dl, dg = dev(gpu, u), dev(gpu, logits), dev(gpu, sgl)
+        dy = gpu.full((1, hidden), 7.0, dtype=gpu.float32, device="cuda")
+        s.moe_layer_verify(0, 1, du.data_ptr(), dl.data_ptr(), dg.data_ptr(), dy.data_ptr())
+        gpu.cuda.synchronize()
+        got = dy.cpu().numpy()
+        idx, w = s.last_route(1)
+        want, widx, ww = oracle_layer(ty, hidden, ff, k, blobs, sh, logits, sgl, u)
+        assert np.array_equal(idx, widx), f"{finite} finite logits"
+        assert np.allclose(w, ww, rtol=2e-6, atol=0)
+        assert rel_l2(got[0], want[0]) <= REL_L2, f"{finite} finite logits: {rel_l2(got[0], want[0])}"
+        monkeypatch.setenv("SHADOWZERO_GGUF_THREE_LAUNCH", "1")
+        dy3 = gpu.zeros((1, hidden), dtype=gpu.float32, device="cuda")
+        s.moe_layer_verify(0, 1, du.data_ptr(), dl.data_ptr(), dg.data_ptr(), dy3.data_ptr())
+        gpu.cuda.synchronize()
+        monkeypatch.delenv("SHADOWZERO_GGUF_THREE_LAUNCH")
+        assert rel_l2(dy3.cpu().numpy()[0], got[0]) <= 2e-7, f"{finite} finite logits: the two forms differ"
+        idx3, w3 = s.last_route(1)
+        assert np.array_equal(idx3, idx) and np.allclose(w3, w, rtol=2e-7, atol=0)
+
+
 @pytest.mark.parametrize("ty", [sz.EXL3(3), sz.IQ3_S])
 def test_moe_layer_with_masked_experts_matches_the_oracle(gpu, ty):
     """Logits of -inf (the reference masks the experts it skips that way, session.rs:6205): a row with fewer finite logits than
