@@ -189,6 +189,38 @@ int32_t sz_verify_accept(const uint32_t* ids, const uint32_t* drafts, uint32_t n
  * draft (drafts[k], *n_drafts of them; 0 when nothing matches).  Host arrays. */
 int32_t sz_lookup_draft(const uint32_t* hist, uint64_t n_hist, uint32_t k, const uint32_t* lens, uint32_t n_lens, uint32_t* drafts,
                         uint32_t* n_drafts);
+
+/* ---- the drafters that need no second model, and the policy that picks a round's window (host code; (f) of the path's callers) --
+ * The suffix drafter (crates/shadowzero-serve/src/engine.rs:844-1015 SuffixDrafter): every trigram of the pushed tokens
+ * remembers the last four places it ended.  propose: among those places for the trigram the sequence ends in, the one whose
+ * match backwards is longest (at most max_match tokens, the more recent on a tie, at least min_match: 0 = the drafter's own,
+ * never under 3); the up to max_k tokens that followed it are the draft.  `extra` (n_extra may be 0) is a neural drafter's
+ * proposal that goes behind the history for the question only (propose_after, engine.rs:998): the index keeps what was pushed. */
+typedef struct sz_suffix_drafter sz_suffix_drafter;
+sz_suffix_drafter* sz_suffix_drafter_new(uint32_t min_match, uint32_t max_match, uint32_t capacity_tokens);
+void sz_suffix_drafter_free(sz_suffix_drafter*);
+int32_t sz_suffix_drafter_extend(sz_suffix_drafter*, const uint32_t* tokens, uint32_t n);          /* push / extend, engine.rs:929-951 */
+uint64_t sz_suffix_drafter_len(const sz_suffix_drafter*);
+int32_t sz_suffix_drafter_propose(sz_suffix_drafter*, const uint32_t* extra, uint32_t n_extra, uint32_t max_k, uint32_t min_match,
+                                  uint32_t* drafts, uint32_t* n_drafts, uint32_t* match_len);
+/* The draft policy (engine.rs:1017-1311 DraftPolicy): running means of a round's cost by its number of rows t (1 + drafts,
+ * at most 8) and of the tokens a neural window yields, decayed counts of kept and refused looked-up drafts by match length.
+ *   neural_k      how many drafts to ask the neural drafter for (base_spec, one more after full windows, 2 after empty ones)
+ *   choose        neural window of t_neural rows, or a lookup window (*lookup = 1) of *t rows out of lookup_k available drafts
+ *   chain         how many of k_avail looked-up tokens to put behind a neural window whose drafts all hold with p_neural
+ *   observe       what a round did: lookup or neural, its rows t, accepted drafts, the lookup's match length, its time
+ *   observe_chain the same for a chained round (t_neural rows of the neural window, then k_chain looked-up tokens) */
+typedef struct sz_draft_policy sz_draft_policy;
+sz_draft_policy* sz_draft_policy_new(uint32_t max_t, uint32_t base_spec, double margin);
+void sz_draft_policy_free(sz_draft_policy*);
+uint32_t sz_draft_policy_neural_k(const sz_draft_policy*, uint32_t rem_tokens);
+int32_t sz_draft_policy_choose(const sz_draft_policy*, uint32_t t_neural, uint32_t lookup_k, uint32_t match_len, int32_t* lookup, uint32_t* t);
+uint32_t sz_draft_policy_chain(const sz_draft_policy*, uint32_t t_neural, double p_neural, uint32_t k_avail, uint32_t match_len);
+int32_t sz_draft_policy_observe(sz_draft_policy*, int32_t lookup, uint32_t t, uint32_t accepted, uint32_t match_len, double round_ms);
+int32_t sz_draft_policy_observe_chain(sz_draft_policy*, uint32_t t_neural, uint32_t k_chain, uint32_t accepted, uint32_t match_len, double round_ms);
+/* For tests and logs: the running acceptance, the rounds seen, cost_ms(t) for t = 1..8, and the kept-rate of looked-up and of
+ * chained drafts for the four match-length classes (any pointer may be null). */
+int32_t sz_draft_policy_state(const sz_draft_policy*, double* accept_ema, double* rounds, double* cost_ms8, double* lookup_rate4, double* chain_rate4);
 /* ---- the rollback point of a speculative pass: device state saved and put back, one launch each way.
  * The reference keeps the recurrent layers' states of a session in a device-side snapshot that it takes again before
  * every pass (GpuSession::snapshot_again, crates/shadowzero-cuda/src/session.rs:3407-3452) and restores when drafts are

@@ -1067,8 +1067,11 @@ def test_activation_quantization_on_the_gpu_is_bit_exact(gpu):
 @pytest.mark.parametrize("tokens,hidden,ff,ne,k,shared,skew", [(48, 512, 256, 16, 4, True, True), (130, 256, 256, 8, 3, False, True),
                                                                  (5, 2048, 512, 40, 10, True, False)])
 def test_prefill_chunk_matches_the_int8_oracle(gpu, tokens, hidden, ff, ne, k, shared, skew):
-    """Routing ids and int8 activation codes bit-exact; the layer output within 1e-3 relative L2 of the oracle that runs the same
-    int8 arithmetic (cpu_expert.rs:243-339 with per-32 activation blocks)."""
+    """Routing ids and the int8 codes of the input activations bit-exact; the layer output within 1e-3 relative L2 of the oracle
+    that runs the same int8 arithmetic (cpu_expert.rs:243-339 with per-32 activation blocks).  The codes of H = silu(gate) * up,
+    quantized again between the two products, are held to a relaxed bar on purpose: at most 1e-3 of them may differ from the
+    oracle's (by one step each), because the device's expf and the fused multiply-add that folds a sub-block's int32 sum into
+    the f32 total leave H a last bit or two away from the oracle's, which now and then crosses a rounding boundary."""
     rng = np.random.default_rng(tokens * 3 + ne)
     ty = sz.IQ3_S
     dbuf, stride, blobs, sh = build_layer(gpu, rng, ty, hidden, ff, ne, shared)
@@ -1109,7 +1112,7 @@ def test_prefill_chunk_matches_the_int8_oracle(gpu, tokens, hidden, ff, ne, k, s
             out, _ = O.expert_int8(sh, hidden, ff, wq, wd)
             acc = acc + np.float32(1.0 / (1.0 + np.exp(-np.float64(sgl[j])))) * out
         assert rel_l2(got[j], acc) <= REL_L2, f"token {j}: {rel_l2(got[j], acc)}"
-    # H codes: the same rounding rule on values that agree to the last bit or two of f32 (device expf against libm's)
+    # H codes: the same rounding rule on values that agree to the last bit or two of f32 (device expf against libm's, fused fold)
     assert code_diff <= 1e-3 * code_total, f"{code_diff} of {code_total} H codes differ"
 
 
