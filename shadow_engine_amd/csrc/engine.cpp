@@ -457,19 +457,27 @@ int head_argmax_rows(sz_session* s, uint32_t n, uint64_t u, uint64_t logits, uin
     return launch("argmax_merge_parts", n, 1, 1, 256, 0, stream, b);
 }
 
-// The matrix-core head: all m <= 8 rows in one pass over the matrix.
-bool head_mfma_ok(const sz_session* s) {
+// The matrix-core head: all m <= 8 rows in one pass over the matrix.  The number of waves a workgroup (each owns at most
+// 512 columns of a row): 4 up to 2048 columns, 6 up to 3072, 8 up to 4096; 0: the shape goes to the scalar kernel.
+uint32_t head_mfma_waves(const sz_session* s) {
     static const bool off = std::getenv("SHADOWZERO_HEAD_SCALAR") != nullptr;
     const sz_session_config& c = s->cfg;
-    return !off && s->head_type == SZ_TYPE_Q8_0 && c.hidden % 256 == 0 && c.hidden <= 2048 && (s->head_w & 15) == 0 && c.vocab >= 16;
+    if (off || s->head_type != SZ_TYPE_Q8_0 || (s->head_w & 15) != 0 || c.vocab < 16) return 0;
+    if (c.hidden % 256 == 0 && c.hidden <= 2048) return 4;
+    if (c.hidden % 192 == 0 && c.hidden <= 3072) return 6;
+    if (c.hidden % 256 == 0 && c.hidden <= 4096) return 8;
+    return 0;
 }
+bool head_mfma_ok(const sz_session* s) { return head_mfma_waves(s) != 0; }
 
 int head_argmax_mfma(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uint64_t ids, uint64_t stream) {
     const sz_session_config& c = s->cfg;
+    const uint32_t waves = head_mfma_waves(s);
     const uint32_t tiles = (c.vocab + 15) / 16;
-    const uint32_t nparts = std::min<uint32_t>(tiles, 512);       // two workgroups a CU (70 KB of LDS each)
+    const uint32_t nparts = std::min<uint32_t>(tiles, waves == 4 ? 512 : 256);       // two workgroups a CU (70 KB of LDS each), one for the wider rows
     const sz_arg a[] = {P(s->head_w), P(u), U32(c.hidden), P(logits), U32(c.vocab), P(s->head_part.ptr), U32(c.vocab), U32(c.hidden), U32(m)};
-    if (launch("head_q8_0_argmax_mfma", nparts, 1, 1, 256, 0, stream, a)) return 1;
+    const char* name = waves == 4 ? "head_q8_0_argmax_mfma" : waves == 6 ? "head_q8_0_argmax_mfma_w6" : "head_q8_0_argmax_mfma_w8";
+    if (launch(name, nparts, 1, 1, 64 * waves, 0, stream, a)) return 1;
     const sz_arg b[] = {P(s->head_part.ptr), U32(nparts), U32(8), P(ids), P(0)};
     return launch("argmax_merge_parts", m, 1, 1, 256, 0, stream, b);
 }

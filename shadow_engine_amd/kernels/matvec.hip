@@ -1128,9 +1128,9 @@ extern "C" __global__ void __launch_bounds__(256) head_q8_0_argmax(const u8* w, 
     }
 }
 
-// The same head on the matrix cores, for cols <= 2048 (a multiple of 256), m <= 8 and a 16-byte aligned matrix.
+// The same head on the matrix cores, for W = 4, 6 or 8 waves and cols <= 512 W (a multiple of 64 W), m <= 8 and a 16-byte aligned matrix.
 // A 16-row tile of the matrix (16 x cols / 32 x 34 contiguous bytes) comes into LDS by global-to-LDS loads, the next tile
-// while this one is multiplied.  Wave w owns the quarter k in [w cols / 4, (w + 1) cols / 4) of every row and keeps its
+// while this one is multiplied.  Wave w owns the share k in [w cols / W, (w + 1) cols / W) of every row and keeps its
 // slice of the inputs in registers for the whole launch, as the B operands of v_mfma_f32_16x16x16_f16: with
 // s_j x_j = the input row times the power of two that takes its largest magnitude to [2^14, 2^15), column 2 j holds
 // f16(s_j x_j) and column 2 j + 1 holds f16(s_j x_j - f16(s_j x_j)): the high parts are finite whatever the activations'
@@ -1140,9 +1140,9 @@ extern "C" __global__ void __launch_bounds__(256) head_q8_0_argmax(const u8* w, 
 // are multiplied by 1 / s_j at the end.  The A operand is the tile's
 // codes: a lane takes 4 consecutive codes of row lane % 16, turns each into the f16 1024 + (code ^ 0x80) by putting 0x64
 // above the byte, and subtracts 1152 (exact).  A 32-block's two products are scaled by the block's f16 scale and added to
-// the lane's running sums in f32, block after block in k order; the four waves' sums are added in wave order.
+// the lane's running sums in f32, block after block in k order; the waves' sums are added in wave order.
 // part[(blockIdx.x * 8 + j) * 2] = {value bits, index} of the workgroup's best row for input j (NaN counts as -inf,
-// ties to the lower index).  grid <= tiles (persistent: tile t goes to workgroup t % grid), block 256.
+// ties to the lower index).  grid <= tiles (persistent: tile t goes to workgroup t % grid), block 64 W.
 typedef _Float16 f16x4 __attribute__((ext_vector_type(4)));
 #define HEAD_PITCH(cols) ((cols) / 32 * 34 + 16)   // bytes between a tile's rows in LDS: 16 rows then fall on different banks
 
@@ -1156,32 +1156,38 @@ __device__ __forceinline__ f16x4 head_codes_f16(u32 q) {
     return f16x4{a[0], a[1], b[0], b[1]};
 }
 
-// Requests tile `t` (rows 16 t .. 16 t + 15, clamped to the last row) into the LDS buffer at byte offset `lds`: wave w
-// brings rows 4 w .. 4 w + 3, each as 16-byte pieces (three instructions a row).
+// Requests tile `t` (rows 16 t .. 16 t + 15, clamped to the last row) into the LDS buffer at byte offset `lds`: wave w of W
+// brings rows w, w + W, .., each as 16-byte pieces (ceil(row bytes / 1024) instructions a row).
+template <int W>
 __device__ __forceinline__ void head_tile_issue(const u8* __restrict__ w, u32 rows, u32 rb, u32 t, u32 lds, u32 wave, u32 lane) {
     const u32 pieces = rb / 16;                           // rb is a multiple of 16 here
 #pragma unroll
-    for (int rr = 0; rr < 4; rr++) {
-        const u32 lr = wave * 4 + rr;
-        const u8* src = w + (u64) min(16 * t + lr, rows - 1) * rb;
-        const u32 dst = lds + lr * (rb + 16);
+    for (int rr = 0; rr < (16 + W - 1) / W; rr++) {
+        const u32 lr = wave + W * rr;
+        if (lr < 16) {
+            const u8* src = w + (u64) min(16 * t + lr, rows - 1) * rb;
+            const u32 dst = lds + lr * (rb + 16);
 #pragma unroll
-        for (int c = 0; c < 3; c++)
-            if (c * 64 + lane < pieces) lds_load<16>(src + (c * 64 + lane) * 16, dst + c * 1024);
+            for (int c = 0; c < 5; c++)
+                if (c * 64 < pieces)
+                    if (c * 64 + lane < pieces) lds_load<16>(src + (c * 64 + lane) * 16, dst + c * 1024);
+        }
     }
 }
 
-extern "C" __global__ void __launch_bounds__(256, 2) head_q8_0_argmax_mfma(const u8* w, const float* x, u32 xs, float* logits, u32 ls, u32* part,
-                                                                           u32 rows, u32 cols, u32 m) {
-    __shared__ __attribute__((aligned(16))) u8 tile[2][16 * HEAD_PITCH(2048)];
-    __shared__ float red[4][256];
+// W waves (4, 6 or 8), cols = 512 W at most and a multiple of 64 W.
+template <int W>
+__device__ __forceinline__ void head_mfma_body(const u8* w, const float* x, u32 xs, float* logits, u32 ls, u32* part, u32 rows, u32 cols, u32 m) {
     __shared__ float s_bv[256];
     __shared__ u32 s_bi[256];
-    __shared__ float s_mx[4][8], s_inv[8];   // largest magnitude of a wave's quarter of every input row; the factor that undoes a row's scale
-    const u32 tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    __shared__ float s_mx[W][8], s_inv[8];   // largest magnitude of a wave's share of every input row; the factor that undoes a row's scale
+    const u32 tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const u32 rb = cols / 32 * 34, pitch = rb + 16;
-    const u32 nbw = cols / 128;                           // 32-blocks of a wave's quarter of k (<= 16)
+    const u32 kw = cols / W, nbw = kw / 32;               // a wave's columns, and their 32-blocks (<= 16)
     const u32 n16 = lane & 15, g4 = lane >> 4;
+    __shared__ __attribute__((aligned(16))) u8 tiles_lds[2 * 16 * HEAD_PITCH(512 * W)];   // two tiles, 16 * pitch bytes apart
+    __shared__ float red[W][256];
+    u8* const tile0 = tiles_lds;
     // the wave's slice of the inputs as B operands: B[k = 4 g4 + i][n = n16], n = 2 j + (0: high part, 1: low part)
     f16x4 xb[16][2];
     {
@@ -1189,7 +1195,7 @@ extern "C" __global__ void __launch_bounds__(256, 2) head_q8_0_argmax_mfma(const
         // all 32 loads go out before the first is waited for (clamped to an address that exists where the lane has no
         // input or the block lies past the row: a load behind a branch is waited for on the spot, a round trip each)
         f32x4 raw[16][2];
-        const float* xj = x + (u64) min(j, m - 1) * xs + wave * (cols / 4) + 4 * g4;
+        const float* xj = x + (u64) min(j, m - 1) * xs + wave * kw + 4 * g4;
 #pragma unroll
         for (int b = 0; b < 16; b++)
 #pragma unroll
@@ -1209,8 +1215,11 @@ extern "C" __global__ void __launch_bounds__(256, 2) head_q8_0_argmax_mfma(const
         mxl = fmaxf(mxl, lane_xor<32>(mxl, lane));
         if (g4 == 0 && lowpart == 0) s_mx[wave][j] = mxl;
         __syncthreads();
+        float mxr = s_mx[0][j];
+#pragma unroll
+        for (int v = 1; v < W; v++) mxr = fmaxf(mxr, s_mx[v][j]);
         float scale, inv;
-        pow2_scale_of(f32_bits(fmaxf(fmaxf(s_mx[0][j], s_mx[1][j]), fmaxf(s_mx[2][j], s_mx[3][j]))), scale, inv);
+        pow2_scale_of(f32_bits(mxr), scale, inv);
         if (wave == 0 && g4 == 0 && lowpart == 0) s_inv[j] = inv;
 #pragma unroll
         for (int b = 0; b < 16; b++)
@@ -1230,26 +1239,30 @@ extern "C" __global__ void __launch_bounds__(256, 2) head_q8_0_argmax_mfma(const
             }
     }
     const u32 tiles = (rows + 15) / 16;
-    const u32 lds0 = __builtin_amdgcn_readfirstlane(lds_offset(tile[0])), lds1 = __builtin_amdgcn_readfirstlane(lds_offset(tile[1]));
+    const u32 lds0 = __builtin_amdgcn_readfirstlane(lds_offset(tile0)), lds1 = lds0 + 16 * pitch;
+    // the load instructions a tile costs this wave: its rows (w, w + W, .. < 16) times the 1 KiB pieces of a row
+    const u32 mine = ((16 - wave + W - 1) / W) * ((rb / 16 + 63) / 64);
     float bv = -__builtin_inff();
     u32 bi = 0xffffffffu;
     u32 t = blockIdx.x, it = 0;
-    if (t < tiles) head_tile_issue(w, rows, rb, t, lds0, wave, lane);
+    if (t < tiles) head_tile_issue<W>(w, rows, rb, t, lds0, wave, lane);
     for (; t < tiles; t += gridDim.x, it++) {
         const u32 tn = t + gridDim.x;
-        if (tn < tiles) head_tile_issue(w, rows, rb, tn, (it & 1) ? lds0 : lds1, wave, lane);
-        // this tile's requests of this wave have landed; the next tile's (4 rows x ceil(pieces / 64) instructions, the youngest
-        // in the queue) may stay in flight - unless logits are stored in the loop: a store is not ordered with the loads
+        if (tn < tiles) head_tile_issue<W>(w, rows, rb, tn, (it & 1) ? lds0 : lds1, wave, lane);
+        // this tile's requests of this wave have landed; the next tile's (the youngest in the queue) may stay in flight -
+        // unless logits are stored in the loop: a store is not ordered with the loads
         if (tn < tiles && !logits) {
-            if (rb > 2048) wait_vm<12>();
-            else if (rb > 1024) wait_vm<8>();
-            else wait_vm<4>();
+            if (mine >= 12) wait_vm<12>();
+            else if (mine >= 10) wait_vm<10>();
+            else if (mine >= 8) wait_vm<8>();
+            else if (mine >= 4) wait_vm<4>();
+            else wait_vm<0>();
         } else {
             wait_vm<0>();
         }
         __syncthreads();                                  // ... and every other wave's
-        const u8* tb = tile[it & 1];
-        const u8* arow = tb + n16 * pitch + wave * nbw * 34;      // A: row n16 of the tile, the wave's quarter of k
+        const u8* tb = tile0 + (it & 1) * 16 * pitch;
+        const u8* arow = tb + n16 * pitch + wave * nbw * 34;      // A: row n16 of the tile, the wave's share of k
         const u8* drow = tb + (4 * g4) * pitch + wave * nbw * 34;  // scales: rows 4 g4 + r
         float tot[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
@@ -1271,12 +1284,11 @@ extern "C" __global__ void __launch_bounds__(256, 2) head_q8_0_argmax_mfma(const
 #pragma unroll
         for (int r = 0; r < 4; r++) red[wave][(4 * g4 + r) * 16 + n16] = tot[r];
         __syncthreads();
-        {
-            // thread (row = tid / 16, n = tid % 16): the four waves' sums in wave order, then high part + low part
+        if (tid < 256) {
+            // thread (row = tid / 16, n = tid % 16): the waves' sums in wave order, then high part + low part
             float s = red[0][tid];
-            s += red[1][tid];
-            s += red[2][tid];
-            s += red[3][tid];
+#pragma unroll
+            for (int v = 1; v < W; v++) s += red[v][tid];
             const float o = lane_xor<1>(s, lane);
             const u32 n = tid & 15, j = n >> 1, row = 16 * t + (tid >> 4);
             if ((n & 1) == 0 && j < m && row < rows) {
@@ -1288,8 +1300,10 @@ extern "C" __global__ void __launch_bounds__(256, 2) head_q8_0_argmax_mfma(const
         }
     }
     // the workgroup's best row per input: thread (row slot tid / 16, n) holds the best of its row slot
-    s_bv[tid] = bv;
-    s_bi[tid] = bi;
+    if (tid < 256) {
+        s_bv[tid] = bv;
+        s_bi[tid] = bi;
+    }
     __syncthreads();
     if (tid < 8) {
         float v = -__builtin_inff();
@@ -1298,6 +1312,21 @@ extern "C" __global__ void __launch_bounds__(256, 2) head_q8_0_argmax_mfma(const
         part[((u64) blockIdx.x * 8 + tid) * 2] = f32_bits(v);
         part[((u64) blockIdx.x * 8 + tid) * 2 + 1] = i;
     }
+}
+
+extern "C" __global__ void __launch_bounds__(256, 2) head_q8_0_argmax_mfma(const u8* w, const float* x, u32 xs, float* logits, u32 ls, u32* part,
+                                                                           u32 rows, u32 cols, u32 m) {
+    head_mfma_body<4>(w, x, xs, logits, ls, part, rows, cols, m);
+}
+// The same for rows of up to 3072 columns (6 waves, block 384) and up to 4096 (8 waves, block 512): a wave still owns at
+// most 512 columns, the tiles take all of a CU's LDS but for a workgroup's share, so one workgroup a CU.
+extern "C" __global__ void __launch_bounds__(384) head_q8_0_argmax_mfma_w6(const u8* w, const float* x, u32 xs, float* logits, u32 ls, u32* part,
+                                                                           u32 rows, u32 cols, u32 m) {
+    head_mfma_body<6>(w, x, xs, logits, ls, part, rows, cols, m);
+}
+extern "C" __global__ void __launch_bounds__(512) head_q8_0_argmax_mfma_w8(const u8* w, const float* x, u32 xs, float* logits, u32 ls, u32* part,
+                                                                           u32 rows, u32 cols, u32 m) {
+    head_mfma_body<8>(w, x, xs, logits, ls, part, rows, cols, m);
 }
 
 // ids[j] = index of the largest of row j's `nparts` partial maxima part[(p * ts + j) * 2] (ties to the lower index).

@@ -646,7 +646,8 @@ def planted_head(rng, vocab, hidden, m, winners=None):
 
 
 @pytest.mark.parametrize("vocab,m,hidden", [(151936, 4, 2048), (1000, 1, 2048), (4099, 8, 2048), (8, 3, 2048),
-                                            (3001, 5, 3072), (517, 2, 768), (2048, 3, 4096)])   # rows that are not a power of two of 32-weight units
+                                            (3001, 5, 3072), (517, 2, 768), (2048, 3, 4096),    # rows that are not a power of two of 32-weight units
+                                            (20000, 8, 4096), (20000, 7, 3072), (5000, 2, 2304), (5000, 3, 2560)])   # six and eight waves a workgroup
 def test_head_argmax_and_logits_match_the_oracle(gpu, vocab, m, hidden):
     rng = np.random.default_rng(vocab + m)
     w, u = planted_head(rng, vocab, hidden, m, winners=[3] + [int(r) for r in rng.choice(vocab, size=m - 1)] if vocab == 4099 else None)
