@@ -452,7 +452,7 @@ __device__ __forceinline__ void rows_one_chunk(const u8* w, u32 rows, u32 cols, 
     const u32 U = cols / 32, rb = cols / F::QK * F::BB;
     const u32 r0 = blockIdx.x * rpb;
     const u32 nrows = min(rpb, rows - r0);
-    const u32 RG = 64 / U, sub = lane / U, ul = lane % U;
+    const u32 lg = 31u - (u32) __builtin_clz(U), RG = 64u >> lg, sub = lane >> lg, ul = lane & (U - 1);   // U divides 64: a power of two
     float x[32][1];
     unit_from_lds(xs, ul, x);
     for (u32 lr = wv * RG + sub; lr < rpb; lr += 4 * RG) {
@@ -622,20 +622,24 @@ __device__ __forceinline__ float route_weights_chosen(const float* lg, u32 ne, u
     return e != 0xffffffffu ? (float) (mine / tz) : 0.0f;
 }
 
+// floor(x / d) for x < 65536 by one multiplication: `magic` = fast_div_magic(d), 1 <= d < 65536 (the one division, done once).
+__device__ __forceinline__ u32 fast_div_magic(u32 d) { return 0xffffffffu / d + 1u; }
+__device__ __forceinline__ u32 fast_div(u32 x, u32 magic) { return __umulhi(x, magic); }
+
 // Copies `n` spans of `span` bytes into LDS regions of `rs` bytes each (a multiple of 16, at least span + 15): span p starts
 // at global address g0(p) and lands so that its first byte is at byte (g0(p) & 15) of region p, which starts at dynamic LDS
 // byte p * rs; a null g0(p) skips the span.  All the loads of a thread (at most 4: n * rs / 16 <= 1024) are in flight
 // before its first store; a chunk that reaches outside its span is read byte by byte, so nothing outside the spans is touched.
 template <class Addr>
 __device__ __forceinline__ void stage_spans(Addr g0, u32 n, u32 span, u32 rs, u32 tid) {
-    const u32 ch = rs / 16, total = n * ch, nthr = blockDim.x;
+    const u32 ch = rs / 16, total = n * ch, nthr = blockDim.x, mch = fast_div_magic(ch);
     u32x4 v[4];
 #pragma unroll
     for (int r = 0; r < 4; r++) {
         const u32 i = tid + nthr * r;
         v[r] = u32x4{0, 0, 0, 0};
         if (i < total) {
-            const u32 p = i / ch, c = i % ch;
+            const u32 p = fast_div(i, mch), c = i - p * ch;
             const u8* g = g0(p);
             if (g) {
                 const u32 head = (u32) ((u64) g & 15);
@@ -717,7 +721,7 @@ __device__ __forceinline__ void decode_gate_up_gguf(const float* logits, u64 eba
     stage_spans([&](u32 p) { return w + (u64) p * part + (u64) r0 * rb; }, 2, rp * rb, rs, threadIdx.x);
     __syncthreads();       // the rows, and for the shared expert's pairs also s_x and the table
     const u32 hg = (u32) ((u64) (w + (u64) r0 * rb) & 15), hu = rs + (u32) ((u64) (w + (u64) part + (u64) r0 * rb) & 15);
-    const u32 U = hidden / 32, RG = 64 / U, sub = lane / U, ul = lane % U;
+    const u32 U = hidden / 32, lg = 31u - (u32) __builtin_clz(U), RG = 64u >> lg, sub = lane >> lg, ul = lane & (U - 1);   // U divides 64: a power of two
     float x[32][1];
     unit_from_lds(s_x, ul, x);
     float* o = act + (u64) pair * ff + r0;
@@ -767,13 +771,13 @@ __device__ __forceinline__ void decode_down_combine_gguf(u64 ebase, u64 estride,
     };
     // as stage_spans, with every lane fetching the id of its chunk's pair from the lane that holds it
     {
-        const u32 ch = rs / 16, total = S * ch;
+        const u32 ch = rs / 16, total = S * ch, mch = fast_div_magic(ch), mn4 = fast_div_magic(n4);
         u32x4 v[4];
         const u8* src[4];
         u32 lo[4], hd[4];
 #pragma unroll
         for (int r = 0; r < 4; r++) {
-            const u32 i = min(tid + nthr * r, total - 1), p = i / ch;
+            const u32 i = min(tid + nthr * r, total - 1), p = fast_div(i, mch);
             const u8* g = nullptr;
             // (p differs between the lanes of a wave: every lane fetches its pair's id from the lane that holds it)
             if (p >= G) g = (const u8*) (shbase + 2 * (u64) part + (u64) r0 * rb);
@@ -781,7 +785,7 @@ __device__ __forceinline__ void decode_down_combine_gguf(u64 ebase, u64 estride,
             if (p < G && e != 0xffffffffu) g = (const u8*) (ebase + e * estride + 2 * (u64) part + (u64) r0 * rb);
             src[r] = g;
             hd[r] = (u32) ((u64) g & 15);
-            lo[r] = (i % ch) * 16;
+            lo[r] = (i - p * ch) * 16;
         }
 #pragma unroll
         for (int r = 0; r < 4; r++) {
@@ -806,7 +810,7 @@ __device__ __forceinline__ void decode_down_combine_gguf(u64 ebase, u64 estride,
         for (int h = 0; h < 8; h++) {
             const u32 i = tid + nthr * h;
             if (i < pieces) {
-                const u32 p = i / n4, q = i % n4;
+                const u32 p = fast_div(i, mn4), q = i - p * n4;
                 *(f32x4*) (s_act + (p * U + q / 8) * XU_PITCH + (q % 8) * 4) = av[h];
             }
         }
@@ -817,7 +821,7 @@ __device__ __forceinline__ void decode_down_combine_gguf(u64 ebase, u64 estride,
         }
     }
     __syncthreads();
-    const u32 RG = 64 / U, sub = lane / U, ul = lane % U;
+    const u32 lg = 31u - (u32) __builtin_clz(U), RG = 64u >> lg, sub = lane >> lg, ul = lane & (U - 1);   // U divides 64: a power of two
     for (u32 p = wave; p < S; p += nthr / 64) {
         const u8* g = row_of(p);
         if (!g) continue;                       // a masked rank: nothing was staged and nothing is added

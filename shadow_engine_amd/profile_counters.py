@@ -13,6 +13,7 @@ workload of bench.py, ARGS its flags (`--workload W`, nothing for the default on
     rocprofv3 --pmc WRITE_SIZE -d D/write -o run -- python3 bench.py ARGS --steps 2 --warmup 1 --no-cpu-baseline --no-other-configs --copy-calibration 1073741824
     rocprofv3 --pmc SQ_INSTS_VALU SQ_ACTIVE_INST_VALU SQ_BUSY_CYCLES SQ_WAVES SQ_WAVE_CYCLES SQ_WAIT_INST_ANY SQ_INSTS_SALU SQ_INSTS_LDS -d D/sq -o run -- python3 bench.py ARGS --steps 2 --warmup 1 --no-cpu-baseline --no-other-configs
     rocprofv3 --pmc SQ_INSTS_MFMA SQ_VALU_MFMA_BUSY_CYCLES SQ_LDS_BANK_CONFLICT SQ_ACTIVE_INST_LDS SQ_INSTS_VMEM_RD SQ_WAIT_ANY SQ_ACTIVE_INST_ANY SQ_INSTS_VMEM_WR -d D/sq2 -o run -- python3 bench.py ARGS --steps 2 --warmup 1 --no-cpu-baseline --no-other-configs
+    rocprofv3 --pmc TCC_HIT_sum TCC_MISS_sum TCC_REQ_sum TCC_EA0_RDREQ_sum -d D/l2 -o run -- python3 bench.py ARGS --steps 2 --warmup 1 --no-cpu-baseline --no-other-configs
 
 then, in the same session (the databases are large and are not kept):
 
@@ -27,7 +28,7 @@ import sqlite3
 import sys
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-OURS = ("verify_", "head_", "argmax_merge", "copy_", "matvec_", "route_", "swiglu", "moe_", "prefill_", "quant_act", "scatter_", "exl3_", "topk_")
+OURS = ("verify_", "decode_", "head_", "argmax_merge", "copy_", "matvec_", "route_", "swiglu", "moe_", "prefill_", "quant_act", "scatter_", "exl3_", "topk_")
 NAMES = {"config5": ("verify_round_config5", "the default benchmark workload (config 5: 48-layer verify round on a 4-row batch, mixed EXL3 K in {2,3,4}, Q8_0 lm_head)", ""),
          "config3": ("verify_layer_and_head_config3", "bench.py --workload config3 (one EXL3 K=3 MoE layer for 4 tokens + Q8_0 head + acceptance)", " --workload config3"),
          "config1": ("matvec_q8_0_config1", "bench.py --workload config1 (one Q8_0 1024 x 2048 matrix-vector product)", " --workload config1"),
@@ -38,6 +39,7 @@ NAMES = {"config5": ("verify_round_config5", "the default benchmark workload (co
          "snapshot": ("copy_ranges_snapshot", "bench.py --workload snapshot (73 device ranges saved and put back)", " --workload snapshot")}
 SQ1 = "SQ_INSTS_VALU SQ_ACTIVE_INST_VALU SQ_BUSY_CYCLES SQ_WAVES SQ_WAVE_CYCLES SQ_WAIT_INST_ANY SQ_INSTS_SALU SQ_INSTS_LDS"
 SQ2 = "SQ_INSTS_MFMA SQ_VALU_MFMA_BUSY_CYCLES SQ_LDS_BANK_CONFLICT SQ_ACTIVE_INST_LDS SQ_INSTS_VMEM_RD SQ_WAIT_ANY SQ_ACTIVE_INST_ANY SQ_INSTS_VMEM_WR"
+L2 = "TCC_HIT_sum TCC_MISS_sum TCC_REQ_sum TCC_EA0_RDREQ_sum"
 TAIL = " --no-cpu-baseline --no-other-configs"
 SHADER_ENGINES = 32          # SQ_BUSY_CYCLES is summed over the 32 shader engines (8 XCDs x 4)
 SIMDS = 1024
@@ -161,6 +163,20 @@ def sq_summary(d, title, args):
         for k in kernels:
             if k in c2:
                 out.append("%-26s " % k + " ".join("%14d" % c2[k].get(n, (0, 0, 0))[1] for n in names))
+    third = os.path.join(d, "l2", "run_results.db")
+    if os.path.exists(third):
+        c3 = pmc(third)
+        out += ["", "The L2 caches (summed over the 8 XCDs' channels), averages a launch:",
+                "  rocprofv3 --pmc %s -d %s/W/l2 -o run -- python3 bench.py%s --steps 2 --warmup 1%s" % (L2, PROF, args, TAIL),
+                "%-26s %14s %14s %14s %14s %9s" % ("kernel", "TCC_REQ", "TCC_HIT", "TCC_MISS", "EA0_RDREQ", "hit rate")]
+        for k in kernels:
+            v = c3.get(k)
+            if not v or "TCC_HIT_sum" not in v:
+                continue
+            hit, miss = v["TCC_HIT_sum"][1], v["TCC_MISS_sum"][1]
+            rate = hit / (hit + miss) if hit + miss else 0.0
+            out.append("%-26s %14d %14d %14d %14d %8.1f%%" % (k, v.get("TCC_REQ_sum", (0, 0, 0))[1], hit, miss, v.get("TCC_EA0_RDREQ_sum", (0, 0, 0))[1], 100 * rate))
+            kernels[k]["l2_hit_rate"] = round(rate, 4)
     return "\n".join(out) + "\n", kernels
 
 
@@ -171,6 +187,13 @@ def main(prof, out_dir):
     os.makedirs(out_dir, exist_ok=True)
     counters = {"kernel_keys": sz.program_keys(), "made_by": "python3 -m shadow_engine_amd.profile_counters (commands in its docstring and in profiles/*.txt)",
                 "peaks": {"simds": SIMDS, "cycles_per_wave64_vector_instruction": 4}, "workloads": {}}
+    try:
+        # workloads summarised earlier on the same kernel sources stay; a file of other sources is started afresh
+        before = json.load(open(os.path.join(out_dir, "counters.json")))
+        if before.get("kernel_keys") == counters["kernel_keys"]:
+            counters["workloads"] = before.get("workloads", {})
+    except (OSError, ValueError):
+        pass
     for wl in sorted(os.listdir(prof)):
         d = os.path.join(prof, wl)
         if wl not in NAMES or not os.path.isdir(d):
