@@ -827,13 +827,10 @@ int32_t sz_moe_prefill_chunk(sz_session* s, uint32_t l, uint32_t tokens, uint64_
         return 1;
     const uint64_t sh = shared ? L.eaddr.ptr + 3ull * c.n_expert * 8 : 0;
     {
+        // routing and quantization do not depend on each other: one launch
         const uint64_t n = T * c.hidden;
-        const sz_arg a[] = {P(x), U64(n), P(pb.xq.ptr), P(pb.xd.ptr)};
-        if (launch("quant_act_q8", (uint32_t) ((n / 32 + 255) / 256), 1, 1, 256, 0, stream, a)) return 1;
-    }
-    {
-        const sz_arg a[] = {P(rl), P(pb.tidx.ptr), P(pb.w.ptr), U32(c.n_expert), U32(c.top_k), U32(tokens)};
-        if (launch("route_topk_rows", (tokens + 3) / 4, 1, 1, 256, 0, stream, a)) return 1;
+        const sz_arg a[] = {P(x), U64(n), P(pb.xq.ptr), P(pb.xd.ptr), P(rl), P(pb.tidx.ptr), P(pb.w.ptr), U32(c.n_expert), U32(c.top_k), U32(tokens)};
+        if (launch("prefill_front", (tokens + 3) / 4 + (uint32_t) ((n / 32 + 255) / 256), 1, 1, 256, 0, stream, a)) return 1;
     }
     const uint64_t items_d = pb.items.ptr + (1 + 2 * max_items) * 4;   // the down kernel's items: runs of up to 32 pairs (PF_TOK_D)
     {

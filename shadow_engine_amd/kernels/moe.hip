@@ -49,6 +49,8 @@ extern "C" __global__ void __launch_bounds__(256) moe_combine_qwen_rows(float* y
 
 // ------------------------------------------------------------------------------------------------ router + planner
 // Routing alone: tidx[j*k + t], weights[j*k + t] (f32), one wave a token.  grid = ceil(m / 4), block 256; ne <= 512, k <= 16.
+// The weights are ex_t over the sum of the chosen ex (route_weights_chosen): a prefill chunk routes thousands of tokens, and
+// the sum over all experts that cancels out of them is 512 f64 exponentials a token.
 extern "C" __global__ void __launch_bounds__(256) route_topk_rows(const float* logits, u32* tidx, float* weights, u32 ne, u32 k, u32 m) {
     __shared__ double exs[4][512];
     __shared__ u32 tops[4][16];
@@ -59,7 +61,7 @@ extern "C" __global__ void __launch_bounds__(256) route_topk_rows(const float* l
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
     u32 count;
-    const float wt = route_weights(logits + (u64) j * ne, ne, k, lane, tops[w], &count);
+    const float wt = route_weights_chosen(logits + (u64) j * ne, ne, k, lane, tops[w], &count);
     if (lane < k) {
         tidx[(u64) j * k + lane] = tops[w][lane];
         weights[(u64) j * k + lane] = wt;

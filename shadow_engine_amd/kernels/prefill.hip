@@ -20,11 +20,8 @@
 
 typedef int i32x4 __attribute__((ext_vector_type(4)));
 
-// q[i] = clamp(round(x[i] / d)), d[b] = amax / 127 over each 32 values (cpu_expert_avx512.rs:25-42).  One thread a block.
-// grid = ceil(n / 32 / 256), block 256.
-extern "C" __global__ void __launch_bounds__(256) quant_act_q8(const float* x, u64 n, i8* q, float* d) {
-    const u64 b = (u64) blockIdx.x * 256 + threadIdx.x;
-    if (b >= n / 32) return;
+// q[i] = clamp(round(x[i] / d)), d[b] = amax / 127 over each 32 values (cpu_expert_avx512.rs:25-42).  One thread a block of 32.
+__device__ __forceinline__ void quant_block_q8(const float* x, u64 b, i8* q, float* d) {
     const f32x4* p = (const f32x4*) (x + b * 32);
     float v[32];
 #pragma unroll
@@ -55,6 +52,39 @@ extern "C" __global__ void __launch_bounds__(256) quant_act_q8(const float* x, u
     o[0] = u32x4{w[0], w[1], w[2], w[3]};
     o[1] = u32x4{w[4], w[5], w[6], w[7]};
     d[b] = dd;
+}
+
+// grid = ceil(n / 32 / 256), block 256.
+extern "C" __global__ void __launch_bounds__(256) quant_act_q8(const float* x, u64 n, i8* q, float* d) {
+    const u64 b = (u64) blockIdx.x * 256 + threadIdx.x;
+    if (b < n / 32) quant_block_q8(x, b, q, d);
+}
+
+// The two things a chunk needs before its tokens can be grouped, in one launch (they do not depend on each other): the
+// routing of its m tokens (workgroups [0, ceil(m / 4)): a wave a token, as route_topk_rows) and the quantization of its
+// activations (the workgroups after them, as quant_act_q8).  grid = ceil(m / 4) + ceil(n / 32 / 256), block 256.
+extern "C" __global__ void __launch_bounds__(256) prefill_front(const float* x, u64 n, i8* q, float* d, const float* logits, u32* tidx, float* weights,
+                                                                u32 ne, u32 k, u32 m) {
+    __shared__ double exs[4][512];
+    __shared__ u32 tops[4][16];
+    const u32 nr = (m + 3) / 4;
+    if (blockIdx.x >= nr) {
+        const u64 b = (u64) (blockIdx.x - nr) * 256 + threadIdx.x;
+        if (b < n / 32) quant_block_q8(x, b, q, d);
+        return;
+    }
+    const u32 lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const u32 j = blockIdx.x * 4 + w;
+    if (j >= m) return;
+    route_ids(logits + (u64) j * ne, ne, k, lane, exs[w], tops[w]);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    u32 count;
+    const float wt = route_weights_chosen(logits + (u64) j * ne, ne, k, lane, tops[w], &count);
+    if (lane < k) {
+        tidx[(u64) j * k + lane] = tops[w][lane];
+        weights[(u64) j * k + lane] = wt;
+    }
 }
 
 #define PF_TOK 64      // tokens of one work item: PF_TOK / 16 MFMA tiles of 16
@@ -160,20 +190,29 @@ __device__ __forceinline__ void pf_tables(u32 tid) {
 }
 
 // Eight consecutive weights (k = 8 kq .. 8 kq + 7 of sub-block g) of one IQ3_S block at `blk` (LDS, 2-byte aligned) as
-// signed int8, and the sub-block's scale d (1 + 2 s) (cpu_expert.rs:99-110).
-__device__ __forceinline__ u64 iq3s_int8x8(const u8* blk, u32 g, u32 kq, float& sw) {
+// signed int8 (cpu_expert.rs:99-110).
+__device__ __forceinline__ u64 iq3s_int8x8(const u8* blk, u32 g, u32 kq) {
     const u32 j = 8 * g + 2 * kq;                       // index of the first of the two 4-weight groups
     const u32 qs = *(const u16*) (blk + 2 + j);
     const u32 qh = blk[66 + g] >> (2 * kq);
     const u32 signs = blk[74 + 4 * g + kq];
-    const u32 sc = (blk[106 + (g >> 1)] >> (4 * (g & 1))) & 0x0f;
-    sw = f16_to_f32(*(const u16*) blk) * (float) (1 + 2 * sc);
     const u32 g0 = pf_grid[(qs & 0xff) | ((qh & 1u) << 8)], g1 = pf_grid[(qs >> 8) | ((qh & 2u) << 7)];
     // negate the bytes whose sign bit is set: (m ^ mask) + (mask & 1) per byte, magnitudes are at most 15 so nothing carries
     const u64 mask = pf_sign[signs];
     const u32 m0 = (u32) mask, m1 = (u32) (mask >> 32);
     const u32 w0 = (g0 ^ m0) + (m0 & 0x01010101u), w1 = (g1 ^ m1) + (m1 & 0x01010101u);
     return ((u64) w1 << 32) | w0;
+}
+
+// The sub-block scales d (1 + 2 s) of a block: the four lanes that share a row (kq = 0..3) would each work out all eight;
+// instead lane (n, kq) works out the two of the byte it is handed (sub-blocks 2 kq and 2 kq + 1) and leaves them in the wave's
+// own strip sw[8][16] (LDS), where the products read them back (a quarter of the arithmetic, conflict-free reads).
+// A wavefront fence must follow before the strip is read.
+__device__ __forceinline__ void iq3s_scales_to_strip(const u8* blk, u32 n, u32 kq, float* sw) {
+    const float d = f16_to_f32(*(const u16*) blk);
+    const u32 sc = blk[106 + kq];
+    sw[(2 * kq) * 16 + n] = d * (float) (1 + 2 * (sc & 0x0f));
+    sw[(2 * kq + 1) * 16 + n] = d * (float) (1 + 2 * (sc >> 4));
 }
 
 #define PF_KC 256      // k of one staged chunk: one IQ3_S block a row
@@ -225,11 +264,15 @@ __device__ __forceinline__ void pf_issue_w(const u8* __restrict__ w, u32 rb, u32
 // order).  aq, ad: the chunk's activations and their scales; bg, bu, bd: the lane's row's block in LDS.
 template <int T, int TOK>
 __device__ __forceinline__ void pf_products_gu(float (&accg)[PF_TILES][4], float (&accu)[PF_TILES][4], const u8* aq, const float* ad, const u8* bg, const u8* bu,
-                                               u32 n, u32 kq) {
+                                               u32 n, u32 kq, float* sw) {
+    iq3s_scales_to_strip(bg, n, kq, sw);
+    iq3s_scales_to_strip(bu, n, kq, sw + 128);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (u32 g = 0; g < 8; g++) {
-        float swg, swu;
-        const u64 b_g = iq3s_int8x8(bg, g, kq, swg), b_u = iq3s_int8x8(bu, g, kq, swu);
+        const float swg = sw[g * 16 + n], swu = sw[128 + g * 16 + n];
+        const u64 b_g = iq3s_int8x8(bg, g, kq), b_u = iq3s_int8x8(bu, g, kq);
         const u32 col = ((2 * g + (kq >> 1)) ^ n) * 16 + 8 * (kq & 1);   // where this lane's 8 activations of a token lie in its row
 #pragma unroll
         for (int a = 0; a < T; a++) {
@@ -247,11 +290,14 @@ __device__ __forceinline__ void pf_products_gu(float (&accg)[PF_TILES][4], float
     }
 }
 template <int T, int TOK>
-__device__ __forceinline__ void pf_products_d(float (&acc)[TOK / 16][4], const u8* aq, const float* ad, const u8* bd, u32 n, u32 kq) {
+__device__ __forceinline__ void pf_products_d(float (&acc)[TOK / 16][4], const u8* aq, const float* ad, const u8* bd, u32 n, u32 kq, float* sws) {
+    iq3s_scales_to_strip(bd, n, kq, sws);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
 #pragma unroll
     for (u32 g = 0; g < 8; g++) {
-        float sw;
-        const u64 b = iq3s_int8x8(bd, g, kq, sw);
+        const float sw = sws[g * 16 + n];
+        const u64 b = iq3s_int8x8(bd, g, kq);
         const u32 col = ((2 * g + (kq >> 1)) ^ n) * 16 + 8 * (kq & 1);
 #pragma unroll
         for (int a = 0; a < T; a++) {
@@ -276,6 +322,7 @@ extern "C" __global__ void __launch_bounds__(256, 2) prefill_gate_up_iq3_s(const
     constexpr u32 AB = PF_AB(PF_TOK), BUF = AB + 2 * PF_WB + PF_DB(PF_TOK);
     __shared__ __attribute__((aligned(16))) u8 stage[2 * BUF];
     __shared__ u32 s_rows[PF_TOK], s_pairs[PF_TOK];
+    __shared__ float s_sw[4][256];   // a wave's strip of sub-block scales: gate [8][16], up [8][16]
     static_assert(sizeof(stage) >= PF_TOK * 65 * sizeof(float), "H reuses the staging area");
     float (*hs)[65] = (float (*)[65]) stage;
     const u32 tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -320,12 +367,12 @@ extern "C" __global__ void __launch_bounds__(256, 2) prefill_gate_up_iq3_s(const
         const u8* bu = buf + AB + PF_WB + lrow * PF_WS + pf_shift(wu, rb, c, lrow);
         switch ((nt + 15) / 16) {   // straight-line code for the item's number of token tiles: the scheduler overlaps one tile's loads and
                                     // matrix instructions with the scaling of the tile before it
-            case 1: pf_products_gu<1, PF_TOK>(accg, accu, aq, ad, bg, bu, n, kq); break;
+            case 1: pf_products_gu<1, PF_TOK>(accg, accu, aq, ad, bg, bu, n, kq, s_sw[wave]); break;
 #if PF_TILES > 2
-            case 2: pf_products_gu<2, PF_TOK>(accg, accu, aq, ad, bg, bu, n, kq); break;
-            case 3: pf_products_gu<3, PF_TOK>(accg, accu, aq, ad, bg, bu, n, kq); break;
+            case 2: pf_products_gu<2, PF_TOK>(accg, accu, aq, ad, bg, bu, n, kq, s_sw[wave]); break;
+            case 3: pf_products_gu<3, PF_TOK>(accg, accu, aq, ad, bg, bu, n, kq, s_sw[wave]); break;
 #endif
-            default: pf_products_gu<PF_TILES, PF_TOK>(accg, accu, aq, ad, bg, bu, n, kq); break;
+            default: pf_products_gu<PF_TILES, PF_TOK>(accg, accu, aq, ad, bg, bu, n, kq, s_sw[wave]); break;
         }
     }
     __syncthreads();   // the staging area becomes H
@@ -361,6 +408,7 @@ extern "C" __global__ void __launch_bounds__(256, 4) prefill_down_iq3_s(const u6
     constexpr u32 TOK = PF_TOK_D, AB = PF_AB(TOK), BUF = AB + PF_WB + PF_DB(TOK);   // two buffers of a chunk: activations | rows | activation scales
     __shared__ __attribute__((aligned(16))) u8 stage[2 * BUF];
     __shared__ u32 s_pairs[TOK];
+    __shared__ float s_sw[4][128];   // a wave's strip of sub-block scales [8][16]
     const u32 tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const u32 n = lane & 15, kq = lane >> 4;
     const u32 lrow = wave * 16 + n;
@@ -396,8 +444,8 @@ extern "C" __global__ void __launch_bounds__(256, 4) prefill_down_iq3_s(const u6
         const u8* aq = buf;
         const float* ad = (const float*) (buf + AB + PF_WB);
         const u8* bd = buf + AB + lrow * PF_WS + pf_shift(wd + (u64) rbi * 64 * rb, rb, c, lrow);
-        if (nt <= 16) pf_products_d<1, TOK>(acc, aq, ad, bd, n, kq);
-        else pf_products_d<2, TOK>(acc, aq, ad, bd, n, kq);
+        if (nt <= 16) pf_products_d<1, TOK>(acc, aq, ad, bd, n, kq, s_sw[wave]);
+        else pf_products_d<2, TOK>(acc, aq, ad, bd, n, kq, s_sw[wave]);
         if (c + 1 == nc) {   // the row block is complete
             const u32 row = (rb0 + rbi) * 64 + lrow;
 #pragma unroll

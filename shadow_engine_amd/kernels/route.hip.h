@@ -264,3 +264,33 @@ __device__ __attribute__((noinline)) float route_weights(const float* lg, u32 ne
     *count = kk;
     return e != 0xffffffffu ? (float) (mine / tz) : 0.0f;
 }
+
+// The same weights without the sum over all experts: w_t = ex_t / (sum of the chosen ex), which is what the reference's
+// (ex_t / z) / (sum of the chosen ex / z) is before rounding; in f64 the two differ by a few units in the last place at
+// most, far below the f32 the weights are rounded to.  Ten exponentials instead of ne: for a caller with the chosen
+// experts in LDS and a wave to spare but no time.  Lane t < k returns the weight of rank t; *count as route_weights.
+__device__ __forceinline__ float route_weights_chosen(const float* lg, u32 ne, u32 k, u32 lane, const u32* top, u32* count) {
+    float lv[8];
+#pragma unroll
+    for (int q = 0; q < 8; q++) lv[q] = lg[min(q * 64 + lane, ne - 1)];
+    const u32 e = lane < k ? top[lane] : 0xffffffffu;
+    const float le = lg[e != 0xffffffffu ? e : 0];
+    float mx = -3.402823466e+38f;
+#pragma unroll
+    for (int q = 0; q < 8; q++)
+        if (q * 64 + lane < ne) mx = fmaxf(mx, lv[q]);
+    mx = wave_max_f32(mx);
+    const double mine = e != 0xffffffffu ? exp((double) (le - mx)) : 0.0;
+    double tz = 0.0;
+    u32 kk = 0;
+#pragma unroll 1
+    for (u32 t = 0; t < k; t++) {
+        const double v = __shfl(mine, t, SZ_WAVE);
+        if (__shfl(e, t, SZ_WAVE) != 0xffffffffu) {
+            tz += v;
+            kk++;
+        }
+    }
+    *count = kk;
+    return e != 0xffffffffu ? (float) (mine / tz) : 0.0f;
+}
