@@ -454,6 +454,8 @@ def run_moe_layer_case(gpu, ty, hidden, ff, ne, k, m, shared):
     (sz.EXL3_HALF(2), 512, 256, 12, 4, 4),
     (sz.IQ3_S, 2048, 512, 24, 10, 4),
     (sz.Q8_0, 1024, 512, 12, 4, 8),
+    (sz.IQ3_S, 2048, 512, 24, 10, 1),              # one token: the two-launch form, whose first launch also selects all k on a wave of its own
+    (sz.Q8_0, 1024, 512, 12, 4, 1),
 ])
 def test_moe_layer_over_seeds_and_logit_kinds(gpu, ty, hidden, ff, ne, k, m):
     """One set of experts, then several batches against the oracle: normal logits, coarse logits (exact ties, the lower index
