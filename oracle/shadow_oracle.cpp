@@ -10,7 +10,8 @@
 //   IQ3_S dequant          the 8 real IQ3_S blocks with ggml's expected bits (tests/golden/iq3_s_blocks.txt).
 //   EXL3 codebooks         independent numpy float16 arithmetic over all 65,536 states; unit-Gaussian statistics.
 //   EXL3 tile decode       bit-loop decode == 64-bit-window decode (two independent statements), K = 1..8 and halves;
-//                          tile_pos is a bijection.
+//                          tile_pos is a bijection.  The K + 1/2 rates (exl3.rs:150-170): PARITY UNPINNED - the reference
+//                          holds no tensor and no known answer at such a rate; the agreement of the two statements is all there is.
 //   EXL3 reconstruct       recorded sum of squares and first four values of the two real tensors in
 //                          tests/golden/exl3_sample.safetensors.
 //   EXL3 matvec_blob       equals x times the reconstructed matrix (dense f64 product) within 2e-4 of the largest output.
