@@ -496,6 +496,7 @@ def test_moe_layer_over_seeds_and_logit_kinds(gpu, ty, hidden, ff, ne, k, m):
     (sz.EXL3(3), sz.F32, 2048, 512, 48, 10, 4),
     (sz.IQ3_S, sz.BF16, 2048, 512, 32, 10, 3),
     (sz.EXL3(4), sz.F16, 512, 256, 10, 4, 8),
+    (sz.IQ3_S, sz.F32, 2048, 512, 32, 10, 1),      # one token: the router's launch, then the two-launch layer
 ])
 def test_moe_block_with_its_router_matches_the_oracle(gpu, ty, rty, hidden, ff, ne, k, m):
     """Session::moe (forward.rs:1009-1034) from the activations alone: the router and the shared expert's gate product
