@@ -157,6 +157,15 @@ int32_t sz_session_set_layer(sz_session*, uint32_t layer, int32_t expert_type, u
  * multiples of 128; the head of an EXL3 checkpoint, session.rs:7179-7187).  The fused arg-max (sz_head_argmax,
  * sz_verify_round) exists for Q8_0 and EXL3; logits and the top 64 for all three. */
 int32_t sz_session_set_head(sz_session*, int32_t ggml_type, uint64_t w);
+/* The optional, INEXACT 2-bit screen of an EXL3 head for the top-64 hand-off (HeadProxy, session.rs:428-441, built at
+ * session.rs:2631-2674 by exl3_build_q2_proxy_K, kernels/exl3.cu:916-996; used by head_top_at, session.rs:5952-6022): off by
+ * default and after every sz_session_set_head, as the reference's exact mode has it (session.rs:786).  k_blk > 0 builds the
+ * 2-bit copy of the current head (vocab * hidden / 4 bytes + an f16 scale per output and 128 inputs; hidden <= 4096) and
+ * makes sz_head_top score every output with it, compute only the k_blk best 128-output blocks of every row exactly (k_blk
+ * is clamped to [16, vocab / 128] as SHADOWZERO_HEAD_KBLK is, 128 there by default) and take the top 64 among those: the
+ * values are the exact head's bit for bit, but an output outside the chosen blocks cannot appear.  sz_head_argmax,
+ * sz_head_logits and sz_verify_round never use it.  k_blk = 0 turns it off again. */
+int32_t sz_session_set_head_proxy(sz_session*, uint32_t k_blk);
 /* 0: sz_verify_round launches its kernels one by one instead of replaying a captured graph (default 1). */
 int32_t sz_session_set_graph(sz_session*, int32_t enabled);
 /* moe_batch_resident (session.rs:8222): y[m][hidden] = the MoE block of layer l on u[m][hidden], from the router logits
@@ -244,8 +253,10 @@ int32_t sz_copy_ranges(const uint64_t* ranges, uint32_t n, uint64_t stream);
 
 /* The session's batch buffers, for tests and measurements (device addresses; the contents are those of the last call):
  * 0 the plan (chosen experts u32[m][k], weights f32[m][k], counts u32[m] for the fused layers), 1 the split-k partial sums of
- * gate and up, 2 the down products (EXL3 layers); 3 the gate and up rows, 4 the down rows of a GGUF layer's pairs.  0 for any other
- * `which`. */
+ * gate and up, 2 the down products (EXL3 layers); 3 the gate and up rows, 4 the down rows of a GGUF layer's pairs; of the
+ * head's 2-bit screen: 5 the levels, 6 their f16 scales, 7 the rows' int8 codes, 8 their scales, 9 their correction terms, 10 the
+ * block maxima f32[m][vocab / 128], 11 the list of chosen blocks (count, then the blocks ascending), 12 the packed logits of the
+ * listed blocks (rows 128 * min(m * k_use, vocab / 128) apart).  0 for any other `which`. */
 uint64_t sz_session_buffer(sz_session*, int32_t which);
 
 /* A whole verify round over device-resident inputs: for every layer l the MoE block on u[l][m][hidden] with rl[l][m][ne]

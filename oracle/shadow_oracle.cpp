@@ -21,6 +21,12 @@
 //   moe_token              recomputed in numpy from orc_backend_matvec outputs; special cases (k = 1, zero shared gate).
 //   int8 activations       closed form in numpy; int32 dots exact against numpy int64.
 //   argmax/topk/accept     numpy sort on adversarial rows (ties, all equal, -inf, NaN); all four outcomes of K = 3.
+//   2-bit head screen      the gates of the reference's own test (crates/shadowzero-cuda/tests/head_proxy.rs:176-232) on its
+//                          shape: cosine of the block maxima with the exact ones above 0.85, the best row's block chosen,
+//                          the number of chosen blocks in range; a float64 restatement of the scores from the levels'
+//                          values; the rotated matrix against the exact product; the textbook distortion of the optimal
+//                          uniform four-level quantizer of a Gaussian (0.1188 of the variance at a step of 0.9957 sigma);
+//                          the choice of blocks against a plain top-k wherever no residue class holds five of them.
 
 #include "shadow_oracle.h"
 
@@ -662,6 +668,173 @@ int orc_accept(const uint32_t* want, const uint32_t* drafts, int n_drafts) {    
         keep++;
     }
     return keep;
+}
+
+// --------------------------------------------------------- the inexact 2-bit lm_head screen (kernels/exl3.cu:916-987,
+// kernels/forward.cu:4371-4622).  The reference holds this path as CUDA kernels only (off in its exact mode,
+// crates/shadowzero-cuda/src/session.rs:786); what follows restates those kernels' arithmetic operation by operation:
+// the same f32 operations in the same order, fused where they call fmaf, the integer parts as integers.
+
+// One 128-point transform without the 1 / sqrt(128) factor, stages h = 1 .. 64 (exl3.cu:21-30).
+static void wht128_raw(float* v) {
+    for (int h = 1; h < 128; h *= 2)
+        for (int i = 0; i < 128; i += 2 * h)
+            for (int j = i; j < i + h; j++) {
+                const float a = v[j], b = v[j + h];
+                v[j] = a + b;
+                v[j + h] = a - b;
+            }
+}
+
+// exl3_build_q2_proxy (exl3.cu:919-987): every 128 x 128 block (output block ob, input block b) of the matrix in the
+// rotated basis, W_rot[i][c] = (row i of the decoded block, transformed over its 128 outputs) / 128 * svh[c], rounded to
+// f16, is cut to the four levels {-3, -1, 1, 3} * sh with sh = f16(0.5 * 0.9957 * rms) of the output's 128 values of the
+// block.  w_q2 holds 16-byte groups [(ob * 2 n_b + 2 b + hb) * 128 + r] of four words; code of input hb * 64 + wi * 16 +
+// 4 sl + bi sits in word wi at bit 8 bi + 2 sl.  w_sc[(ob * n_b + b) * 128 + r] = sh.
+int orc_q2_proxy_build(uint64_t ni, uint64_t no, int bits, const uint8_t* blob, uint64_t nbytes, uint32_t* w_q2, uint16_t* w_sc) {
+    if (ni % 128 || no % 128 || nbytes != orc_exl3_blob_len(ni, no, bits, 0)) return 2;
+    std::vector<float> w(ni * no);
+    if (orc_exl3_reconstruct(ni, no, bits, 0, 2, blob, nbytes, 1, w.data())) return 2;
+    const size_t n_b = ni / 128, n_ob = no / 128;
+    std::vector<float> svh(no);
+    for (size_t i = 0; i < no; i++) svh[i] = f16_at(blob, 2 * ni + 2 * i);
+    parallel_chunks(n_ob, std::max<size_t>((n_ob + hw_threads() - 1) / hw_threads(), 1), [&](size_t first, size_t last) {
+        std::vector<uint16_t> wh(128 * 128);   // [output][input]
+        float row[128];
+        for (size_t ob = first; ob < last; ob++)
+            for (size_t b = 0; b < n_b; b++) {
+                for (size_t i = 0; i < 128; i++) {
+                    for (size_t c = 0; c < 128; c++) row[c] = w[(b * 128 + i) * no + ob * 128 + c];
+                    wht128_raw(row);
+                    for (size_t c = 0; c < 128; c++) wh[c * 128 + i] = orc_f32_to_f16(row[c] * 0.0078125f * svh[ob * 128 + c]);
+                }
+                for (size_t r = 0; r < 128; r++) {
+                    float sq = 0.0f;
+                    for (size_t c = 0; c < 128; c++) {
+                        const float fv = orc_f16_to_f32(wh[r * 128 + c]);
+                        sq = std::fmaf(fv, fv, sq);
+                    }
+                    const float delta = 0.9957f * std::sqrt(sq * 0.0078125f);
+                    const uint16_t sh = orc_f32_to_f16(0.5f * delta);
+                    const float thr = 2.0f * orc_f16_to_f32(sh);
+                    w_sc[(ob * n_b + b) * 128 + r] = sh;
+                    for (size_t hb = 0; hb < 2; hb++)
+                        for (size_t wi = 0; wi < 4; wi++) {
+                            uint32_t pw = 0;
+                            for (size_t sl = 0; sl < 4; sl++)
+                                for (size_t bi = 0; bi < 4; bi++) {
+                                    const float fv = orc_f16_to_f32(wh[r * 128 + hb * 64 + wi * 16 + sl * 4 + bi]);
+                                    const uint32_t q = fv >= 0.0f ? (fv >= thr ? 3u : 2u) : (fv <= -thr ? 0u : 1u);
+                                    pw |= q << (bi * 8 + sl * 2);
+                                }
+                            w_q2[((ob * (n_b * 2) + b * 2 + hb) * 128 + r) * 4 + wi] = pw;
+                        }
+                }
+            }
+    });
+    return 0;
+}
+
+// exl3_rotate_rows_f32 + proxy_q2_quant_x (exl3.cu:610-625, forward.cu:4376-4420) for one input row: (x * suh) transformed
+// without the 1 / sqrt(128) factor, every 128-block to int8 codes with the scale amax / 127 (round half to even), four codes
+// a word; x_corr = -3 * (sum of the block's codes) * scale.
+void orc_q2_proxy_quant_x(const uint8_t* blob, const float* x, uint64_t ni, uint32_t* xq, float* x_sc, float* x_corr) {
+    float v[128];
+    for (size_t b = 0; b < ni / 128; b++) {
+        for (size_t i = 0; i < 128; i++) v[i] = x[b * 128 + i] * f16_at(blob, 2 * (b * 128 + i));
+        wht128_raw(v);
+        float amax = 0.0f;
+        for (size_t i = 0; i < 128; i++) amax = std::fmax(amax, std::fabs(v[i]));
+        const float sc = amax > 0.0f ? amax / 127.0f : 0.0f;
+        const float inv = sc > 0.0f ? 1.0f / sc : 0.0f;
+        int tot = 0;
+        for (size_t k = 0; k < 32; k++) {
+            uint32_t p4 = 0;
+            for (size_t e = 0; e < 4; e++) {
+                const int q = (int) std::nearbyint(std::fmax(-127.0f, std::fmin(127.0f, v[4 * k + e] * inv)));
+                tot += q;
+                p4 |= (uint32_t) (uint8_t) (int8_t) q << (8 * e);
+            }
+            xq[b * 32 + k] = p4;
+        }
+        x_sc[b] = sc;
+        x_corr[b] = -3.0f * (float) tot * sc;
+    }
+}
+
+// proxy_q2_dp4a_bmax (forward.cu:4428-4497) for one input row: the score of output r is the sum over the input blocks, in
+// order, of fma(sh, fma(2 x_sc, sum of code * u, x_corr), acc) with u = 0..3 the stored level (the level's value is
+// 2 u - 3, which is what the correction term restores); bmax[ob] = the largest score of the block's 128 outputs.
+void orc_q2_proxy_bmax(const uint32_t* w_q2, const uint16_t* w_sc, const uint32_t* xq, const float* x_sc, const float* x_corr,
+                       uint64_t n_ob, uint64_t ni, float* bmax) {
+    const size_t n_b = ni / 128;
+    parallel_chunks(n_ob, std::max<size_t>((n_ob + hw_threads() - 1) / hw_threads(), 1), [&](size_t first, size_t last) {
+        for (size_t ob = first; ob < last; ob++) {
+            float best = 0.0f;
+            for (size_t r = 0; r < 128; r++) {
+                float acc = 0.0f;
+                for (size_t b = 0; b < n_b; b++) {
+                    int ia = 0;
+                    for (size_t hb = 0; hb < 2; hb++)
+                        for (size_t wi = 0; wi < 4; wi++) {
+                            const uint32_t word = w_q2[((ob * (n_b * 2) + b * 2 + hb) * 128 + r) * 4 + wi];
+                            for (size_t sl = 0; sl < 4; sl++) {
+                                const uint32_t xw = xq[b * 32 + hb * 16 + wi * 4 + sl];
+                                for (size_t bi = 0; bi < 4; bi++)
+                                    ia += (int) (int8_t) (xw >> (8 * bi)) * (int) ((word >> (8 * bi + 2 * sl)) & 3u);
+                            }
+                        }
+                    const float wsc = orc_f16_to_f32(w_sc[(ob * n_b + b) * 128 + r]);
+                    acc = std::fmaf(wsc, std::fmaf(2.0f * x_sc[b], (float) ia, x_corr[b]), acc);
+                }
+                best = r == 0 ? acc : std::fmax(best, acc);
+            }
+            bmax[ob] = best;
+        }
+    });
+}
+
+// proxy_pick_rows + proxy_compact_seen (forward.cu:4519-4622): for each of the m rows of bmax[m][n_ob], the blocks i = t,
+// t + 256, .. of each t < 256 give their four best (strictly larger replaces the fourth, equal values keep the earlier
+// block; NaN counts as -3e38), the 1024 candidates are ordered by value descending then block ascending, and the first
+// k_blk that are blocks are marked.  The union of the rows' marks, ascending, goes to sel[1 ..]; sel[0] = their number, at
+// most max_sel.  Returns the number of marked blocks.
+uint32_t orc_q2_proxy_pick(const float* bmax, uint32_t m, uint32_t n_ob, uint32_t k_blk, uint32_t max_sel, uint32_t* sel) {
+    std::vector<uint8_t> seen(n_ob, 0);
+    for (uint32_t row = 0; row < m; row++) {
+        std::vector<std::pair<float, uint32_t>> cand;
+        for (uint32_t t = 0; t < 256; t++) {
+            float lv[4] = {-3.0e38f, -3.0e38f, -3.0e38f, -3.0e38f};
+            uint32_t li[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+            for (uint32_t i = t; i < n_ob; i += 256) {
+                float v = bmax[(size_t) row * n_ob + i];
+                if (v != v) v = -3.0e38f;
+                if (v > lv[3]) {
+                    lv[3] = v;
+                    li[3] = i;
+                    for (int k = 3; k > 0; k--)
+                        if (lv[k] > lv[k - 1] || (lv[k] == lv[k - 1] && li[k] < li[k - 1])) {
+                            std::swap(lv[k], lv[k - 1]);
+                            std::swap(li[k], li[k - 1]);
+                        }
+                }
+            }
+            for (int k = 0; k < 4; k++) cand.push_back({lv[k], li[k]});
+        }
+        std::sort(cand.begin(), cand.end(), [](const std::pair<float, uint32_t>& a, const std::pair<float, uint32_t>& b) {
+            return a.first > b.first || (a.first == b.first && a.second < b.second);
+        });
+        for (uint32_t t = 0; t < k_blk && t < n_ob && t < cand.size(); t++)
+            if (cand[t].second < n_ob) seen[cand[t].second] = 1;
+    }
+    uint32_t n = 0;
+    for (uint32_t ob = 0; ob < n_ob; ob++)
+        if (seen[ob]) {
+            if (n < max_sel) sel[1 + n] = ob;
+            n++;
+        }
+    sel[0] = n < max_sel ? n : max_sel;
+    return n;
 }
 
 }   // extern "C"

@@ -123,6 +123,18 @@ void orc_topk(const float* row, size_t n, int k, float* vals, uint32_t* ids);
 int orc_lookup_draft(const uint32_t* hist, size_t n_hist, int k, const uint32_t* lens, int n_lens, uint32_t* out);
 int orc_accept(const uint32_t* want, const uint32_t* drafts, int n_drafts);
 
+/* ---- the inexact 2-bit lm_head screen: kernels/exl3.cu:916-987 (builder), kernels/forward.cu:4371-4622 (input codes,
+ * block maxima, choice of blocks).  The reference has these as CUDA kernels only; their arithmetic is restated. ---------- */
+/* w_q2: no/128 * ni/128 * 2 * 128 groups of four u32; w_sc: no * ni/128 f16 bit patterns. */
+int orc_q2_proxy_build(uint64_t ni, uint64_t no, int bits, const uint8_t* blob, uint64_t nbytes, uint32_t* w_q2, uint16_t* w_sc);
+/* One input row: xq[ni/4] packed int8 codes, x_sc[ni/128], x_corr[ni/128]. */
+void orc_q2_proxy_quant_x(const uint8_t* blob, const float* x, uint64_t ni, uint32_t* xq, float* x_sc, float* x_corr);
+/* One input row: bmax[n_ob] = the largest screen score of every 128-output block. */
+void orc_q2_proxy_bmax(const uint32_t* w_q2, const uint16_t* w_sc, const uint32_t* xq, const float* x_sc, const float* x_corr,
+                       uint64_t n_ob, uint64_t ni, float* bmax);
+/* bmax[m][n_ob] -> sel[0] = number of chosen blocks (at most max_sel), sel[1 ..] the blocks ascending; returns the number marked. */
+uint32_t orc_q2_proxy_pick(const float* bmax, uint32_t m, uint32_t n_ob, uint32_t k_blk, uint32_t max_sel, uint32_t* sel);
+
 int orc_hardware_threads(void);
 
 #ifdef __cplusplus

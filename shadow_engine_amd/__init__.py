@@ -144,6 +144,7 @@ _SIGNATURES = {
     "sz_session_free": (None, [_vp]),
     "sz_session_set_layer": (_i32, [_vp, _u32, _i32, _u64, _u64, _i32, _u64]),
     "sz_session_set_head": (_i32, [_vp, _i32, _u64]),
+    "sz_session_set_head_proxy": (_i32, [_vp, _u32]),
     "sz_session_set_graph": (_i32, [_vp, _i32]),
     "sz_moe_layer_verify": (_i32, [_vp, _u32, _u32, _u64, _u64, _u64, _u64, _u64]),
     "sz_session_set_router": (_i32, [_vp, _u32, _i32, _u64, _i32, _u64]),
@@ -507,11 +508,15 @@ class Session:
     def set_head(self, ggml_type, w_dev):
         check(lib().sz_session_set_head(self._h, ggml_type, w_dev))
 
+    def set_head_proxy(self, k_blk):
+        """Build (k_blk > 0) or drop (0) the inexact 2-bit screen of the EXL3 head that head_top then uses."""
+        check(lib().sz_session_set_head_proxy(self._h, k_blk))
+
     def set_graph(self, enabled):
         check(lib().sz_session_set_graph(self._h, int(enabled)))
 
     def buffer(self, which):
-        """Device address of a batch buffer: 0 plan, 1 gate/up partial sums, 2 down products."""
+        """Device address of a batch buffer: 0 plan, 1 gate/up partial sums, 2 down products, 3/4 GGUF rows, 5..12 the head screen's."""
         return lib().sz_session_buffer(self._h, which)
 
     def moe_layer_verify(self, layer, m, u_dev, rl_dev, sgl_dev, y_dev, stream=0):

@@ -297,6 +297,11 @@ struct sz_session {
     DevBuf plan, eg, act, eo, part, dn, head_part, logits, topv, topi, topo, ids;
     DevBuf head_xa, head_inv;   // an EXL3 head's rotated inputs as f16 high and low parts (16 rows of 128 a 128-block), and the tokens' scales
     DevBuf rl, sgl;   // the router's outputs for a batch: f32[max_rows][n_expert], f32[max_rows]
+    // the optional 2-bit screen of an EXL3 head (HeadProxy of session.rs:428-441): k_blk = 0 is off
+    struct {
+        uint32_t k_blk = 0;
+        DevBuf w_q2, w_sc, xq, x_sc, x_corr, bmax, seen, sel, logits;
+    } hp;
     struct {
         DevBuf xq, xd, tidx, w, cnt, offs, list, items, hq, hd, eo;
     } pf;   // the prefill chunk's buffers, grown on demand
@@ -503,11 +508,55 @@ int head_exl3(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uint64_t i
     }
     const uint32_t nparts = c.vocab / 128, lds = 4 * ((kbs + 3) / 4) * ((m + 1) / 2) * 1024;
     const std::string kn = "head_exl3_" + std::to_string(bits);
-    const sz_arg a[] = {P(s->head_w), P(s->head_xa.ptr), P(s->head_inv.ptr), P(logits), U32(c.vocab), P(s->head_part.ptr), U32(c.hidden), U32(c.vocab), U32(m)};
+    const sz_arg a[] = {P(s->head_w), P(s->head_xa.ptr), P(s->head_inv.ptr), P(logits), U32(c.vocab), P(s->head_part.ptr), U32(c.hidden), U32(c.vocab), U32(m), P(0)};
     if (launch(kn.c_str(), nparts, 1, 1, 256, lds, stream, a)) return 1;
     if (!ids) return 0;
     const sz_arg b[] = {P(s->head_part.ptr), U32(nparts), U32(8), P(ids), P(0)};
     return launch("argmax_merge_parts", m, 1, 1, 256, 0, stream, b);
+}
+
+// The number of blocks a row may choose for a hand-off of need_k values (session.rs:5961): three quarters of k_blk, at least
+// 64, when only a few are needed.
+uint32_t head_proxy_k_use(const sz_session* s, uint32_t need_k) {
+    const uint32_t k = s->hp.k_blk;
+    return need_k <= 16 ? std::min(std::max(k * 3 / 4, 64u), k) : k;
+}
+
+// The screened head (mv_head_proxy_sparse, session.rs:5952-5995): rotate the rows, their int8 codes, the block maxima of the
+// 2-bit copy, the k_use best blocks of every row, their union as a list, and the exact head on the listed blocks only.
+// Leaves the list in hp.sel and the packed logits (rows max_sel * 128 apart) in hp.logits; *max_sel_out = the list's bound.
+int head_proxy_sparse(sz_session* s, uint32_t m, uint64_t u, uint32_t need_k, uint32_t* max_sel_out, uint64_t stream) {
+    const sz_session_config& c = s->cfg;
+    const uint32_t kbs = c.hidden / 128, n_ob = c.vocab / 128, bits = (uint32_t) s->head_type - 1020;
+    const uint32_t k_use = head_proxy_k_use(s, need_k), max_sel = std::min(m * k_use, n_ob);
+    {
+        const sz_arg a[] = {P(s->head_w), P(u), U32(c.hidden), P(s->head_xa.ptr), P(s->head_inv.ptr), U32(c.hidden)};
+        if (launch("exl3_head_rotate", m, 1, 1, 64 * std::min<uint32_t>(16, kbs), 0, stream, a)) return 1;
+    }
+    {
+        const sz_arg a[] = {P(s->head_w), P(u), U32(c.hidden), P(s->hp.xq.ptr), P(s->hp.x_sc.ptr), P(s->hp.x_corr.ptr), U32(c.hidden)};
+        if (launch("proxy_q2_quant_x", kbs, m, 1, 64, 0, stream, a)) return 1;
+    }
+    {
+        const sz_arg a[] = {P(s->hp.w_q2.ptr), P(s->hp.w_sc.ptr), P(s->hp.xq.ptr), P(s->hp.x_sc.ptr), P(s->hp.x_corr.ptr), P(s->hp.bmax.ptr),
+                            U32(n_ob), U32(c.hidden), U32(m)};
+        if (launch(m == 1 ? "proxy_q2_bmax_m1" : m <= 4 ? "proxy_q2_bmax_m4" : "proxy_q2_bmax_m8", n_ob, 1, 1, 128, 0, stream, a)) return 1;
+    }
+    {
+        const sz_arg a[] = {P(s->hp.bmax.ptr), U32(n_ob), U32(k_use), P(s->hp.seen.ptr)};
+        if (launch("proxy_pick_rows", m, 1, 1, 256, 0, stream, a)) return 1;
+    }
+    {
+        const sz_arg a[] = {P(s->hp.seen.ptr), U32(n_ob), U32(max_sel), P(s->hp.sel.ptr)};
+        if (launch("proxy_compact_seen", 1, 1, 1, 64, 0, stream, a)) return 1;
+    }
+    const uint32_t lds = 4 * ((kbs + 3) / 4) * ((m + 1) / 2) * 1024;
+    const std::string kn = "head_exl3_" + std::to_string(bits);
+    const sz_arg a[] = {P(s->head_w), P(s->head_xa.ptr), P(s->head_inv.ptr), P(s->hp.logits.ptr), U32(max_sel * 128), P(s->head_part.ptr),
+                        U32(c.hidden), U32(c.vocab), U32(m), P(s->hp.sel.ptr)};
+    if (launch(kn.c_str(), max_sel, 1, 1, 256, lds, stream, a)) return 1;
+    *max_sel_out = max_sel;
+    return 0;
 }
 
 int head_argmax(sz_session* s, uint32_t m, uint64_t u, uint64_t ids, uint64_t stream) {
@@ -666,14 +715,47 @@ int32_t sz_session_set_head(sz_session* s, int32_t ty, uint64_t w) {
     }
     s->head_type = ty;
     s->head_w = w;
+    s->hp.k_blk = 0;   // a screen belongs to the head it was built from
     for (auto& g : s->graphs) sz_graph_destroy(g.second);
     s->graphs.clear();
     return 0;
 }
 
+int32_t sz_session_set_head_proxy(sz_session* s, uint32_t k_blk) {
+    clear_error();
+    if (!s) return fail("sz_session_set_head_proxy: null session");
+    if (k_blk == 0) {
+        s->hp.k_blk = 0;
+        return 0;
+    }
+    const sz_session_config& c = s->cfg;
+    if (!head_is_exl3(s)) return fail("sz_session_set_head_proxy: the screen is built from an EXL3 head (set one first)");
+    if (c.hidden > 4096) return fail("sz_session_set_head_proxy: hidden above 4096");      // session.rs:2656
+    const uint64_t n_ob = c.vocab / 128, n_b = c.hidden / 128, rows = 8;
+    const uint32_t k = (uint32_t) std::min<uint64_t>(std::max<uint32_t>(k_blk, 16), n_ob);   // session.rs:2659
+    const uint64_t max_sel = std::min<uint64_t>(rows * k, n_ob);
+    if ((max_sel * 128 + 4095) / 4096 > 64) return fail("sz_session_set_head_proxy: 8 rows of k_blk blocks are more than the top-64 merge takes (k_blk <= 256)");
+    auto& h = s->hp;
+    if (h.w_q2.need((uint64_t) c.vocab * c.hidden / 4) || h.w_sc.need((uint64_t) c.vocab * n_b * 2) || h.xq.need(rows * n_b * 32 * 4) ||
+        h.x_sc.need(rows * n_b * 4) || h.x_corr.need(rows * n_b * 4) || h.bmax.need(rows * n_ob * 4) || h.seen.need((n_ob + 31) / 32 * 4) ||
+        h.sel.need((1 + max_sel) * 4) || h.logits.need(rows * max_sel * 128 * 4))
+        return 1;
+    if (sz_memset(h.seen.ptr, 0, h.seen.bytes, 0) || sz_memset(h.xq.ptr, 0, h.xq.bytes, 0) || sz_memset(h.x_sc.ptr, 0, h.x_sc.bytes, 0) ||
+        sz_memset(h.x_corr.ptr, 0, h.x_corr.bytes, 0))
+        return 1;
+    const std::string kn = "exl3_build_q2_proxy_" + std::to_string(s->head_type - 1020);
+    const sz_arg a[] = {P(s->head_w), P(h.w_q2.ptr), P(h.w_sc.ptr), U32(c.hidden), U32(c.vocab)};
+    if (launch(kn.c_str(), (uint32_t) n_ob, (uint32_t) n_b, 1, 256, 0, 0, a)) return 1;
+    if (sz_stream_synchronize(0)) return 1;
+    h.k_blk = k;
+    return 0;
+}
+
 uint64_t sz_session_buffer(sz_session* s, int32_t which) {
     if (!s) return 0;
-    return which == 0 ? s->plan.ptr : which == 1 ? s->part.ptr : which == 2 ? s->dn.ptr : which == 3 ? s->eg.ptr : which == 4 ? s->eo.ptr : 0;
+    const uint64_t at[] = {s->plan.ptr, s->part.ptr, s->dn.ptr, s->eg.ptr, s->eo.ptr, s->hp.w_q2.ptr, s->hp.w_sc.ptr, s->hp.xq.ptr, s->hp.x_sc.ptr,
+                           s->hp.x_corr.ptr, s->hp.bmax.ptr, s->hp.sel.ptr, s->hp.logits.ptr};
+    return which >= 0 && which < (int32_t) (sizeof at / sizeof at[0]) ? at[which] : 0;
 }
 
 int32_t sz_session_set_graph(sz_session* s, int32_t enabled) {
@@ -719,6 +801,18 @@ int32_t sz_head_top(sz_session* s, uint32_t m, uint64_t u, uint32_t* top_host, u
     const uint32_t nb = (c.vocab + 4095) / 4096;
     if (nb > 64) return fail("sz_head_top: vocabulary above 262144");
     if (head_check(s, m, u, "sz_head_top")) return 1;
+    if (s->hp.k_blk) {   // head_top_at, session.rs:5997-6022: the screened form, the top 64 among the chosen blocks
+        if (s->topv.need(8ull * 64 * 64 * 4) || s->topi.need(8ull * 64 * 64 * 4) || s->topo.need(8ull * 128 * 4)) return 1;
+        uint32_t max_sel = 0;
+        if (head_proxy_sparse(s, m, u, 64, &max_sel, stream)) return 1;
+        const uint32_t nbs = (max_sel * 128 + 4095) / 4096;
+        const sz_arg a[] = {P(s->hp.logits.ptr), U32(max_sel * 128), P(s->hp.sel.ptr), U32(nbs), P(s->topv.ptr), P(s->topi.ptr)};
+        if (launch("topk_slices_blks", m * nbs, 1, 1, 256, 0, stream, a)) return 1;
+        const sz_arg b[] = {P(s->topv.ptr), P(s->topi.ptr), U32(nbs), P(s->topo.ptr)};
+        if (launch("topk_merge", m, 1, 1, 256, 0, stream, b)) return 1;
+        if (sz_stream_synchronize(stream)) return 1;
+        return sz_download(top_host, s->topo.ptr, (uint64_t) m * 128 * 4);
+    }
     if (s->logits.need((uint64_t) c.max_rows * c.vocab * 4) || s->topv.need((uint64_t) c.max_rows * nb * 64 * 4) ||
         s->topi.need((uint64_t) c.max_rows * nb * 64 * 4) || s->topo.need((uint64_t) c.max_rows * 128 * 4))
         return 1;

@@ -136,8 +136,9 @@ __device__ __forceinline__ void wht_stage(float& v0, float& v1, u32 lane) {
 }
 
 // 128-point Walsh-Hadamard transform inside one wave: the lane holds elements `lane` (v0) and `lane + 64` (v1).  Stages
-// h = 1, 2, .. 32 cross lanes, h = 64 is the lane's own pair; then the 1/sqrt(128) factor (exl3.rs:583-599).
-__device__ __forceinline__ void wht128_wave(float& v0, float& v1, u32 lane) {
+// h = 1, 2, .. 32 cross lanes, h = 64 is the lane's own pair; then the 1/sqrt(128) factor (exl3.rs:583-599), which the
+// raw form leaves out.
+__device__ __forceinline__ void wht128_wave_raw(float& v0, float& v1, u32 lane) {
     wht_stage<1>(v0, v1, lane);
     wht_stage<2>(v0, v1, lane);
     wht_stage<4>(v0, v1, lane);
@@ -145,8 +146,14 @@ __device__ __forceinline__ void wht128_wave(float& v0, float& v1, u32 lane) {
     wht_stage<16>(v0, v1, lane);
     wht_stage<32>(v0, v1, lane);
     const float a = v0 + v1, b = v0 - v1;
-    v0 = a * 0.08838835f;
-    v1 = b * 0.08838835f;
+    v0 = a;
+    v1 = b;
+}
+
+__device__ __forceinline__ void wht128_wave(float& v0, float& v1, u32 lane) {
+    wht128_wave_raw(v0, v1, lane);
+    v0 *= 0.08838835f;
+    v1 *= 0.08838835f;
 }
 
 // The decode loop of one wave: the 8 tile rows of input block kb against the M rotated inputs in the wave's strip xw
@@ -868,17 +875,23 @@ extern "C" __global__ void __launch_bounds__(1024) exl3_head_rotate(const u8* bl
 // from xa once, in units of 4 rows) sit in LDS.  The four waves' sums are added in wave order, scaled back, taken through
 // the output-side transform and scales, optionally stored as logits[j * ls + column], and the block's best column of every
 // row goes to part[(ob * 8 + j) * 2] = {value bits, column} (a NaN counts as -inf, ties to the lower column).
-// grid = out / 128, block 256, dynamic LDS = 4 * ceil(in / 512) * ceil(m / 2) KiB.
+// With a block list (sel[0] = n, sel[1 ..] = blocks; matvec_cols_exl3_pre_sparse of the reference, exl3.cu tail) workgroup
+// i < n takes block sel[1 + i] and its logits and best go to place i instead of ob: logits[j * ls + 128 i + column in block];
+// the arithmetic of a block does not depend on which workgroup runs it, so these are the bits the full pass gives.
+// grid = out / 128 (or the list's bound), block 256, dynamic LDS = 4 * ceil(in / 512) * ceil(m / 2) KiB.
 template <int K>
 __device__ __forceinline__ void exl3_head_kernel(const u8* __restrict__ blob, const u16* __restrict__ xa, const float* __restrict__ inv,
-                                                 float* __restrict__ logits, u32 ls, u32* __restrict__ part, u32 in_f, u32 out_f, u32 m) {
+                                                 float* __restrict__ logits, u32 ls, u32* __restrict__ part, u32 in_f, u32 out_f, u32 m,
+                                                 const u32* __restrict__ sel) {
     constexpr int D = 4;
     typedef Exl3Rows<K, D> R;
     constexpr int stride = R::stride, ur = R::unit_rows;
     constexpr bool one_shift = 16 + 3 * K <= 32;
     extern __shared__ __attribute__((aligned(16))) u16 a_sh[];            // [wave][its blocks][4 nq A rows][128]; afterwards the waves' sums
     __shared__ __attribute__((aligned(16))) u32 wb_all[4][R::words];
-    const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, ob = blockIdx.x;
+    const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, at = blockIdx.x;
+    if (sel && at >= sel[0]) return;                                       // a list shorter than the grid
+    const u32 ob = sel ? sel[1 + at] : at;
     const u32 kbs = in_f / 128, nkbw = (kbs + 3) / 4, nq = (m + 1) / 2;
     const u32 nkb = wave < kbs ? (kbs - wave + 3) / 4 : 0;                 // this wave's blocks: wave, wave + 4, ..
     const u32 nr = nkb * 8;
@@ -1016,8 +1029,8 @@ __device__ __forceinline__ void exl3_head_kernel(const u8* __restrict__ blob, co
         v1 *= sv1;
         const u32 c0 = ob * 128 + lane, c1 = c0 + 64;
         if (logits) {
-            logits[(u64) j * ls + c0] = v0;
-            logits[(u64) j * ls + c1] = v1;
+            logits[(u64) j * ls + at * 128 + lane] = v0;
+            logits[(u64) j * ls + at * 128 + lane + 64] = v1;
         }
         float bv = v0 != v0 ? -__builtin_inff() : v0;
         u32 bi = c0;
@@ -1035,16 +1048,137 @@ __device__ __forceinline__ void exl3_head_kernel(const u8* __restrict__ blob, co
             argmax_merge(bv, bi, ov, oi);
         }
         if (lane == 0) {
-            part[((u64) ob * 8 + j) * 2] = f32_bits(bv);
-            part[((u64) ob * 8 + j) * 2 + 1] = bi;
+            part[((u64) at * 8 + j) * 2] = f32_bits(bv);
+            part[((u64) at * 8 + j) * 2 + 1] = bi;
         }
+    }
+}
+
+// ------------------------------------------------------------------------------------------ the 2-bit screen of the head
+// An inexact, optional shortcut of the reference for the top-64 hand-off (exl3.cu:916-987, forward.cu:4371-4497,
+// session.rs:5952-5995): a 2-bit copy of the head in the rotated basis scores every output cheaply, only the best 128-output
+// blocks are then computed exactly.  Built once a head.  Block (ob, b) = outputs ob * 128 .., inputs b * 128 ..: the decoded
+// weights of an input row are transformed over the block's 128 outputs (no 1/sqrt(128) here nor on the inputs: 1/128 once),
+// times svh, rounded to f16; an output's 128 values of the block are then cut to the levels {-3, -1, 1, 3} * sh, sh = f16(0.5
+// * 0.9957 * rms) (the optimal uniform four-level step of a Gaussian), the level u = 0..3 stored in two bits: the 16-byte
+// group [(ob * 2 n_b + 2 b + hb) * 128 + r] holds inputs hb * 64 .. + 63 of output r, word wi bit 8 bi + 2 sl = input
+// hb * 64 + 16 wi + 4 sl + bi (a byte lane a dot-product-of-four operand after a shift and a mask).  w_sc[(ob * n_b + b) * 128 + r] = sh.
+// grid = (out / 128, in / 128), block 256.
+template <int K>
+__device__ __forceinline__ void exl3_q2_proxy_build(const u8* __restrict__ blob, u32* __restrict__ w_q2, u16* __restrict__ w_sc, u32 in_f, u32 out_f) {
+    __shared__ _Float16 ws[4][16][130];       // a wave's tile row as decoded (f16 values): [input row][output]
+    __shared__ u16 wh[128][130];              // the block in the rotated basis as f16: [output][input]
+    const u32 wave = threadIdx.x >> 6, lane = threadIdx.x & 63, ob = blockIdx.x, b = blockIdx.y;
+    const u32 n_b = in_f / 128, nt = out_f / 16;
+    const u32* tr = (const u32*) (blob + 2 * (u64) in_f + 2 * (u64) out_f + 4);
+    const u16* svh = (const u16*) (blob + 2 * (u64) in_f) + ob * 128;
+    const float sv0 = f16_to_f32(svh[lane]), sv1 = f16_to_f32(svh[lane + 64]);
+    const u32 col = (lane >> 3) * 16 + (lane & 7);
+    for (u32 kk = wave; kk < 8; kk += 4) {
+        u32 S[EXL3_NW(K, false)];
+        exl3_load_words<K>(tr, nt, b * 8 + kk, ob, lane, S);
+        f16x2 w[16];
+        exl3_decode32<K>(S, w);
+#pragma unroll
+        for (int i = 0; i < 32; i++) ws[wave][EXL3_ROW(i)][col + 8 * EXL3_HALF(i)] = w[i / 2][i % 2];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        for (u32 r = 0; r < 16; r++) {
+            float v0 = (float) ws[wave][r][lane], v1 = (float) ws[wave][r][lane + 64];
+            wht128_wave_raw(v0, v1, lane);
+            // the product rounded to f32 first, then to f16, as the reference's two operations do: left to itself the compiler
+            // makes one multiply-and-convert instruction of them, which rounds once and differs where the f32 product is an
+            // f16 tie
+            float p0 = v0 * 0.0078125f * sv0, p1 = v1 * 0.0078125f * sv1;
+            asm volatile("" : "+v"(p0), "+v"(p1));
+            wh[lane][kk * 16 + r] = __builtin_bit_cast(u16, (_Float16) p0);
+            wh[lane + 64][kk * 16 + r] = __builtin_bit_cast(u16, (_Float16) p1);
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    }
+    __syncthreads();
+    if (threadIdx.x < 128) {
+        const u32 r = threadIdx.x;
+        float sq = 0.0f;
+        for (u32 c = 0; c < 128; c++) {
+            const float fv = f16_to_f32(wh[r][c]);
+            sq = __builtin_fmaf(fv, fv, sq);
+        }
+        // the f32 square root correctly rounded, as the reference's sqrtf is: the f64 root of an f32 rounds to it (53 >= 2 * 24 + 2
+        // bits); the single-precision instruction is an ulp off now and then
+        const float delta = 0.9957f * (float) __builtin_sqrt((double) (sq * 0.0078125f));
+        const u16 sh = __builtin_bit_cast(u16, (_Float16) (0.5f * delta));
+        const float thr = 2.0f * f16_to_f32(sh);
+        w_sc[((u64) ob * n_b + b) * 128 + r] = sh;
+        for (u32 hb = 0; hb < 2; hb++) {
+            u32x4 words;
+#pragma unroll
+            for (u32 wi = 0; wi < 4; wi++) {
+                u32 pw = 0;
+#pragma unroll
+                for (u32 sl = 0; sl < 4; sl++)
+#pragma unroll
+                    for (u32 bi = 0; bi < 4; bi++) {
+                        const float fv = f16_to_f32(wh[r][hb * 64 + wi * 16 + sl * 4 + bi]);
+                        const u32 q = fv >= 0.0f ? (fv >= thr ? 3u : 2u) : (fv <= -thr ? 0u : 1u);
+                        pw |= q << (bi * 8 + sl * 2);
+                    }
+                words[wi] = pw;
+            }
+            ((u32x4*) w_q2)[((u64) ob * (n_b * 2) + b * 2 + hb) * 128 + r] = words;
+        }
+    }
+}
+
+// The rows of a batch for the screen (exl3_rotate_rows_f32 + proxy_q2_quant_x of the reference: exl3.cu:610-625,
+// forward.cu:4376-4420): block b of row j, (x * suh) transformed without the 1/sqrt(128) factor, as int8 codes with the
+// scale amax / 127 (round half to even), four codes a word: xq[(j * n_b + b) * 32 + w] = inputs 4 w .. 4 w + 3 of the block;
+// x_sc = the scale, x_corr = -3 * (sum of the codes) * scale (the levels are 2 u - 3 and the screen multiplies by u).
+// grid = (in / 128, m), block 64.
+extern "C" __global__ void __launch_bounds__(64) proxy_q2_quant_x(const u8* blob, const float* x, u32 xs, u32* xq, float* x_sc, float* x_corr, u32 in_f) {
+    const u32 lane = threadIdx.x, b = blockIdx.x, j = blockIdx.y, n_b = in_f / 128;
+    const u16* suh = (const u16*) blob + b * 128;
+    const float* xj = x + (u64) j * xs + b * 128;
+    float v0 = xj[lane] * f16_to_f32(suh[lane]), v1 = xj[lane + 64] * f16_to_f32(suh[lane + 64]);
+    wht128_wave_raw(v0, v1, lane);
+    const float amax = wave_max_f32(fmaxf(__builtin_fabsf(v0), __builtin_fabsf(v1)));
+    const float sc = amax > 0.0f ? amax / 127.0f : 0.0f;
+    const float inv = sc > 0.0f ? 1.0f / sc : 0.0f;
+    const i32 q0 = (i32) __builtin_rintf(fmaxf(-127.0f, fminf(127.0f, v0 * inv)));
+    const i32 q1 = (i32) __builtin_rintf(fmaxf(-127.0f, fminf(127.0f, v1 * inv)));
+    u32 p0 = ((u32) q0 & 0xffu) << (8 * (lane & 3)), p1 = ((u32) q1 & 0xffu) << (8 * (lane & 3));
+    p0 |= f32_bits(lane_xor<1>(bits_f32(p0), lane));
+    p1 |= f32_bits(lane_xor<1>(bits_f32(p1), lane));
+    p0 |= f32_bits(lane_xor<2>(bits_f32(p0), lane));
+    p1 |= f32_bits(lane_xor<2>(bits_f32(p1), lane));
+    u32* o = xq + ((u64) j * n_b + b) * 32;
+    if ((lane & 3) == 0) {
+        o[lane >> 2] = p0;
+        o[16 + (lane >> 2)] = p1;
+    }
+    i32 tot = q0 + q1;
+    tot += (i32) f32_bits(lane_xor<1>(bits_f32((u32) tot), lane));
+    tot += (i32) f32_bits(lane_xor<2>(bits_f32((u32) tot), lane));
+    tot += (i32) f32_bits(lane_xor<4>(bits_f32((u32) tot), lane));
+    tot += (i32) f32_bits(lane_xor<8>(bits_f32((u32) tot), lane));
+    tot += (i32) f32_bits(lane_xor<16>(bits_f32((u32) tot), lane));
+    tot += (i32) f32_bits(lane_xor<32>(bits_f32((u32) tot), lane));
+    if (lane == 0) {
+        x_sc[(u64) j * n_b + b] = sc;
+        x_corr[(u64) j * n_b + b] = -3.0f * (float) tot * sc;
     }
 }
 
 #define EXL3_HEAD_ENTRIES(K)                                                                                                          \
     extern "C" __global__ void __launch_bounds__(256) head_exl3_##K(const u8* blob, const u16* xa, const float* inv, float* logits, u32 ls, \
-                                                                     u32* part, u32 in_f, u32 out_f, u32 m) {                             \
-        exl3_head_kernel<K>(blob, xa, inv, logits, ls, part, in_f, out_f, m);                                                         \
+                                                                     u32* part, u32 in_f, u32 out_f, u32 m, const u32* sel) {             \
+        exl3_head_kernel<K>(blob, xa, inv, logits, ls, part, in_f, out_f, m, sel);                                                    \
+    }                                                                                                                                 \
+    extern "C" __global__ void __launch_bounds__(256) exl3_build_q2_proxy_##K(const u8* blob, u32* w_q2, u16* w_sc, u32 in_f, u32 out_f) { \
+        exl3_q2_proxy_build<K>(blob, w_q2, w_sc, in_f, out_f);                                                                        \
     }
 EXL3_HEAD_ENTRIES(1)
 EXL3_HEAD_ENTRIES(2)

@@ -180,10 +180,11 @@ extern "C" __global__ void __launch_bounds__(256) route_plan_res_small(const flo
 // Bitonic sort of 4096 (value, id) pairs in LDS, value descending then id ascending; a NaN counts as -inf.
 __device__ __forceinline__ bool tk_before(float va, u32 ia, float vb, u32 ib) { return va > vb || (va == vb && ia < ib); }
 
-__device__ __forceinline__ void tk_sort4096(float* v, u32* id, u32 tid) {
-    for (u32 size = 2; size <= 4096; size <<= 1) {
+template <u32 N>
+__device__ __forceinline__ void tk_sort_pow2(float* v, u32* id, u32 tid) {
+    for (u32 size = 2; size <= N; size <<= 1) {
         for (u32 stride = size >> 1; stride > 0; stride >>= 1) {
-            for (u32 t = tid; t < 2048; t += 256) {
+            for (u32 t = tid; t < N / 2; t += 256) {
                 const u32 lo = (t / stride) * 2 * stride + (t % stride), hi = lo + stride;
                 const bool desc = (lo & size) == 0;   // this run sorts best-first
                 const float va = v[lo], vb = v[hi];
@@ -200,6 +201,8 @@ __device__ __forceinline__ void tk_sort4096(float* v, u32* id, u32 tid) {
         }
     }
 }
+
+__device__ __forceinline__ void tk_sort4096(float* v, u32* id, u32 tid) { tk_sort_pow2<4096>(v, id, tid); }
 
 // Slice b of row r (blockIdx.x = r * nb + b): the 64 best of logits[r*stride + 4096 b .. +4096) into sv/si[(r*nb + b)*64 ..].
 // Slots past the vocabulary hold (-inf, 0xffffffff).  grid = rows * nb, block 256.
@@ -238,6 +241,168 @@ extern "C" __global__ void __launch_bounds__(256) topk_merge(const float* sv, co
     if (tid < 64) {
         out[(u64) r * 128 + tid] = f32_bits(v[tid]);
         out[(u64) r * 128 + 64 + tid] = id[tid];
+    }
+}
+
+// ------------------------------------------------------------------------------------------ the 2-bit screen of the head
+// The inexact, optional top-64 path of the reference (forward.cu:4371-4660; off unless asked for): the 2-bit copy of the head
+// that exl3_build_q2_proxy_K made scores every output against the rows' int8 codes (proxy_q2_quant_x), the best score of a
+// 128-output block is its mark, the k_blk best-marked blocks of every row are computed exactly (head_exl3_K with the list)
+// and the top 64 are taken among those.
+//
+// Block ob = blockIdx.x, lane = output r of the block.  The score of r for row j: over the input blocks b in order,
+// acc = fma(sh, fma(2 x_sc[j][b], sum_i code_i * u_i, x_corr[j][b]), acc) — the integer sums are dot-products-of-four of a
+// code word with four levels (the level word shifted by 2 sl and masked gives inputs 4 sl' ..), exact in any order; the
+// f32 part is the reference's, operation by operation.  The rows' codes are the same for every lane (scalar loads).
+// bmax[j * n_ob + ob] = the largest score of the block.  grid = out / 128, block 128.
+template <int M>
+__device__ __forceinline__ void proxy_q2_bmax(const u32* __restrict__ w_q2, const u16* __restrict__ w_sc, const u32* __restrict__ xq,
+                                              const float* __restrict__ x_sc, const float* __restrict__ x_corr, float* __restrict__ bmax,
+                                              u32 n_ob, u32 in_f, u32 m) {
+    __shared__ float s_mx[2][M];
+    const u32 ob = blockIdx.x, r = threadIdx.x, n_b = in_f / 128;
+    const u32x4* wq = (const u32x4*) w_q2 + (u64) ob * n_b * 256 + r;
+    const u16* sc = w_sc + (u64) ob * n_b * 128 + r;
+    float acc[M];
+#pragma unroll
+    for (int j = 0; j < M; j++) acc[j] = 0.0f;
+#pragma unroll 2
+    for (u32 b = 0; b < n_b; b++) {
+        const u32x4 q[2] = {wq[(u64) b * 256], wq[(u64) b * 256 + 128]};
+        const float wsc = f16_to_f32(sc[b * 128]);
+        i32 ia[M];
+#pragma unroll
+        for (int j = 0; j < M; j++) ia[j] = 0;
+#pragma unroll
+        for (int hb = 0; hb < 2; hb++)
+#pragma unroll
+            for (int wi = 0; wi < 4; wi++)
+#pragma unroll
+                for (int sl = 0; sl < 4; sl++) {
+                    const u32 u = (q[hb][wi] >> (2 * sl)) & 0x03030303u;
+#pragma unroll
+                    for (int j = 0; j < M; j++)
+                        ia[j] = __builtin_amdgcn_sdot4((i32) xq[((u64) min((u32) j, m - 1) * n_b + b) * 32 + hb * 16 + wi * 4 + sl], (i32) u, ia[j], false);
+                }
+#pragma unroll
+        for (int j = 0; j < M; j++) {
+            const u64 at = (u64) min((u32) j, m - 1) * n_b + b;
+            acc[j] = __builtin_fmaf(wsc, __builtin_fmaf(2.0f * x_sc[at], (float) ia[j], x_corr[at]), acc[j]);
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < M; j++) {
+        const float mx = wave_max_f32(acc[j]);
+        if ((r & 63) == 0) s_mx[r >> 6][j] = mx;
+    }
+    __syncthreads();
+    if (r < M && r < m) bmax[(u64) r * n_ob + ob] = fmaxf(s_mx[0][r], s_mx[1][r]);
+}
+
+extern "C" __global__ void __launch_bounds__(128) proxy_q2_bmax_m1(const u32* w_q2, const u16* w_sc, const u32* xq, const float* x_sc, const float* x_corr,
+                                                                   float* bmax, u32 n_ob, u32 in_f, u32 m) {
+    proxy_q2_bmax<1>(w_q2, w_sc, xq, x_sc, x_corr, bmax, n_ob, in_f, m);
+}
+extern "C" __global__ void __launch_bounds__(128) proxy_q2_bmax_m4(const u32* w_q2, const u16* w_sc, const u32* xq, const float* x_sc, const float* x_corr,
+                                                                   float* bmax, u32 n_ob, u32 in_f, u32 m) {
+    proxy_q2_bmax<4>(w_q2, w_sc, xq, x_sc, x_corr, bmax, n_ob, in_f, m);
+}
+extern "C" __global__ void __launch_bounds__(128) proxy_q2_bmax_m8(const u32* w_q2, const u16* w_sc, const u32* xq, const float* x_sc, const float* x_corr,
+                                                                   float* bmax, u32 n_ob, u32 in_f, u32 m) {
+    proxy_q2_bmax<8>(w_q2, w_sc, xq, x_sc, x_corr, bmax, n_ob, in_f, m);
+}
+
+// Row j = blockIdx.x: marks the k_blk best blocks of bmax[j][0 .. n_ob) in the bit map `seen` (forward.cu:4519-4563, with its
+// way of choosing: thread t keeps the four best of blocks t, t + 256, .. — a strictly larger value replaces the fourth, so of
+// equal values the earlier block stays; a NaN counts as -3e38 — and the 1024 kept are ordered by value descending, block
+// ascending; a thread that holds five of the k_blk best loses one, as there).  grid = m, block 256.
+extern "C" __global__ void __launch_bounds__(256) proxy_pick_rows(const float* bmax, u32 n_ob, u32 k_blk, u32* seen) {
+    __shared__ float v[1024];
+    __shared__ u32 id[1024];
+    const u32 tid = threadIdx.x;
+    const float* row = bmax + (u64) blockIdx.x * n_ob;
+    float lv[4] = {-3.0e38f, -3.0e38f, -3.0e38f, -3.0e38f};
+    u32 li[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+    for (u32 i = tid; i < n_ob; i += 256) {
+        float x = row[i];
+        if (x != x) x = -3.0e38f;
+        if (x > lv[3]) {
+            lv[3] = x;
+            li[3] = i;
+#pragma unroll
+            for (int k = 3; k > 0; k--)
+                if (tk_before(lv[k], li[k], lv[k - 1], li[k - 1])) {
+                    const float tv = lv[k];
+                    lv[k] = lv[k - 1];
+                    lv[k - 1] = tv;
+                    const u32 ti = li[k];
+                    li[k] = li[k - 1];
+                    li[k - 1] = ti;
+                }
+        }
+    }
+#pragma unroll
+    for (int k = 0; k < 4; k++) {
+        v[tid * 4 + k] = lv[k];
+        id[tid * 4 + k] = li[k];
+    }
+    __syncthreads();
+    tk_sort_pow2<1024>(v, id, tid);
+    for (u32 t = tid; t < k_blk && t < n_ob && t < 1024; t += 256) {
+        const u32 ob = id[t];
+        if (ob < n_ob) atomicOr(&seen[ob >> 5], 1u << (ob & 31));
+    }
+}
+
+// The marked blocks in ascending order into sel[1 ..], their number (at most max_sel; what does not fit is dropped) into
+// sel[0]; the bit map is left cleared for the next call (forward.cu:4577-4622).  One wave: lane l takes words l, l + 64, ..
+// grid 1, block 64.
+extern "C" __global__ void __launch_bounds__(64) proxy_compact_seen(u32* seen, u32 n_ob, u32 max_sel, u32* sel) {
+    const u32 lane = threadIdx.x, n_words = (n_ob + 31) >> 5;
+    u32 base = 0;
+    for (u32 w0 = 0; w0 < n_words; w0 += 64) {
+        const u32 idx = w0 + lane;
+        u32 mask = idx < n_words ? seen[idx] : 0u;
+        if (idx < n_words) seen[idx] = 0u;
+        const u32 cnt = __builtin_popcount(mask);
+        // inclusive prefix sum of cnt over the lanes
+        u32 pref = cnt;
+        for (u32 off = 1; off < 64; off <<= 1) {
+            const u32 o = (u32) __builtin_amdgcn_ds_bpermute((i32) ((lane - off) & 63) * 4, (i32) pref);
+            if (lane >= off) pref += o;
+        }
+        u32 pos = base + pref - cnt;
+        while (mask) {
+            const u32 bit = (u32) __builtin_ctz(mask);
+            mask &= mask - 1;
+            if (pos < max_sel) sel[1 + pos] = idx * 32 + bit;
+            pos++;
+        }
+        base += (u32) __builtin_amdgcn_readlane((i32) pref, 63);
+    }
+    if (lane == 0) sel[0] = min(base, max_sel);
+}
+
+// topk_slices over the packed logits of a block list (forward.cu:4626-4647): element i of row r (i < 128 sel[0]) is output
+// sel[1 + i / 128] * 128 + i % 128; elements past the list hold (-inf, 0xffffffff).  Since the list ascends, packed order is
+// output order and ties go to the lower output as everywhere.  grid = rows * nb, block 256.
+extern "C" __global__ void __launch_bounds__(256) topk_slices_blks(const float* logits, u32 stride, const u32* sel, u32 nb, float* sv, u32* si) {
+    __shared__ float v[4096];
+    __shared__ u32 id[4096];
+    const u32 tid = threadIdx.x, r = blockIdx.x / nb, b = blockIdx.x % nb;
+    const u32 n = sel[0] << 7;
+    for (u32 t = tid; t < 4096; t += 256) {
+        const u32 i = b * 4096 + t;
+        float x = i < n ? logits[(u64) r * stride + i] : -__builtin_inff();
+        if (x != x) x = -__builtin_inff();
+        v[t] = x;
+        id[t] = i < n ? (sel[1 + (i >> 7)] << 7) | (i & 127) : 0xffffffffu;
+    }
+    __syncthreads();
+    tk_sort4096(v, id, tid);
+    if (tid < 64) {
+        sv[(u64) blockIdx.x * 64 + tid] = v[tid];
+        si[(u64) blockIdx.x * 64 + tid] = id[tid];
     }
 }
 

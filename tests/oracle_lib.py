@@ -81,6 +81,10 @@ def lib():
         "orc_topk": (None, [f32p, C.c_size_t, C.c_int, f32p, vp]),
         "orc_accept": (C.c_int, [vp, vp, C.c_int]),
         "orc_hardware_threads": (C.c_int, []),
+        "orc_q2_proxy_build": (C.c_int, [C.c_uint64, C.c_uint64, C.c_int, u8p, C.c_uint64, vp, vp]),
+        "orc_q2_proxy_quant_x": (None, [u8p, f32p, C.c_uint64, vp, f32p, f32p]),
+        "orc_q2_proxy_bmax": (None, [vp, vp, vp, f32p, f32p, C.c_uint64, C.c_uint64, f32p]),
+        "orc_q2_proxy_pick": (C.c_uint32, [f32p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_uint32, vp]),
     }
     for name, (res, args) in sig.items():
         fn = getattr(L, name)
@@ -283,3 +287,45 @@ def lookup_draft(hist, k, lens=(3, 2)):
     L.orc_lookup_draft.argtypes = [C.c_void_p, C.c_size_t, C.c_int, C.c_void_p, C.c_int, C.c_void_p]
     n = L.orc_lookup_draft(_p(hist), hist.size, k, _p(lens), lens.size, _p(out))
     return out[:n].tolist()
+
+
+def q2_proxy_build(inf, outf, bits, blob):
+    """The 2-bit screen of an EXL3 head: (w_q2 u32[outf/128][inf/128][2][128][4], w_sc u16[outf/128][inf/128][128])."""
+    blob = _c(blob, np.uint8)
+    wq = np.zeros((outf // 128, inf // 128, 2, 128, 4), np.uint32)
+    ws = np.zeros((outf // 128, inf // 128, 128), np.uint16)
+    r = lib().orc_q2_proxy_build(inf, outf, bits, _p(blob), blob.size, _p(wq), _p(ws))
+    assert r == 0, r
+    return wq, ws
+
+
+def q2_proxy_quant_x(blob, x, inf):
+    """Rows x[m][inf] -> (xq u32[m][inf/4], x_sc f32[m][inf/128], x_corr f32[m][inf/128])."""
+    blob = _c(blob, np.uint8)
+    x = _c(x, np.float32).reshape(-1, inf)
+    m = x.shape[0]
+    xq = np.zeros((m, inf // 4), np.uint32)
+    sc = np.zeros((m, inf // 128), np.float32)
+    corr = np.zeros((m, inf // 128), np.float32)
+    for j in range(m):
+        lib().orc_q2_proxy_quant_x(_p(blob), _p(x[j]), inf, _p(xq[j]), _p(sc[j]), _p(corr[j]))
+    return xq, sc, corr
+
+
+def q2_proxy_bmax(wq, ws, xq, sc, corr):
+    """bmax f32[m][outf/128] from the screen and the rows' codes."""
+    n_ob, n_b = ws.shape[0], ws.shape[1]
+    m = xq.shape[0]
+    out = np.zeros((m, n_ob), np.float32)
+    for j in range(m):
+        lib().orc_q2_proxy_bmax(_p(wq), _p(ws), _p(xq[j]), _p(sc[j]), _p(corr[j]), n_ob, n_b * 128, _p(out[j]))
+    return out
+
+
+def q2_proxy_pick(bmax, k_blk, max_sel):
+    """The chosen blocks (ascending) of all rows of bmax together, cut to max_sel, and the number marked before the cut."""
+    bmax = _c(bmax, np.float32)
+    m, n_ob = bmax.shape
+    sel = np.zeros(1 + max_sel, np.uint32)
+    n = lib().orc_q2_proxy_pick(_p(bmax), m, n_ob, k_blk, max_sel, _p(sel))
+    return sel[1:1 + int(sel[0])].copy(), int(n)
