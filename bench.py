@@ -14,6 +14,7 @@ lines carry the same fields):
     config3  one EXL3 K=3 MoE layer for 4 tokens + head + acceptance (weights of the one layer stay warm in cache)
     config4  one prefill chunk: 512 tokens through the 512 IQ3_S experts of a layer on int8 activations (int8 MFMA)
     exl3head the 151,936 x 2048 lm_head of an EXL3 checkpoint (--bits K, default 4) for the batch, arg-max fused in
+    exl3top  the same head's top-64 hand-off to the host; --screen N goes through the inexact 2-bit screen, N blocks a row
     stage    one EXL3 layer of a safetensors checkpoint staged into HBM (the loader beside the path; PCIe-inclusive)
     snapshot the rollback point of a pass: 73 device ranges (79 MB of recurrent state) saved and put back, a launch each
 
@@ -250,6 +251,37 @@ def exl3_head(torch, sz, synth, synth_device, stream, bits):
     w.counters_key = "exl3head" if (bits == 4 and ROWS == 4) else None
     w.cpu = ("exl3_matvec", (blob, bits, u[0].cpu().numpy()))
     w.keep = (sess, blob, u, ids)
+    return w
+
+
+def exl3_head_top(torch, sz, synth, synth_device, stream, bits, k_blk):
+    """The top-64 hand-off of an EXL3 head (151936 x 2048): logits, slice sorts and merge, the 2 KiB a row brought to the host;
+    with k_blk > 0 through the inexact 2-bit screen (the k_blk best 128-output blocks a row computed exactly)."""
+    w = Workload()
+    sess = sz.Session(HIDDEN, FF, 8, 2, 0, VOCAB, 8)
+    blob = synth_device.exl3_matrix(torch, 21, HIDDEN, VOCAB, bits)
+    sess.set_head(sz.EXL3(bits), blob.data_ptr())
+    if k_blk:
+        sess.set_head_proxy(k_blk)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(14)
+    u = torch.randn((ROWS, HIDDEN), device="cuda", generator=g)
+    w.step = lambda: sess.head_top(ROWS, u.data_ptr(), stream.handle)
+    screen = VOCAB * HIDDEN // 4 + VOCAB * (HIDDEN // 128) * 2
+    if k_blk:
+        chosen = min(ROWS * min(max(k_blk, 16), VOCAB // 128), VOCAB // 128)
+        w.step_bytes = screen + chosen * 128 * HIDDEN * bits // 8 + ROWS * HIDDEN * 4
+        w.kernel_bytes = {"proxy_q2_bmax_m%d" % (1 if ROWS == 1 else 4 if ROWS <= 4 else 8): screen}
+    else:
+        w.step_bytes = blob.numel() + ROWS * HIDDEN * 4 + 2 * ROWS * VOCAB * 4
+        w.kernel_bytes = {"head_exl3_%d" % bits: blob.numel() + HIDDEN // 128 * 16 * 256 + ROWS * VOCAB * 4}
+    w.dtype = ("int8 x 2-bit dot products (screen), then " if k_blk else "") + "f32 accumulate over EXL3 f16 codebook weights (f16 matrix cores)"
+    w.describe = {"workload": "top-64 hand-off of the EXL3 lm_head 151936 x 2048 at K = %d for %d rows, to the host%s" % (
+        bits, ROWS, " through the inexact 2-bit screen, %d blocks a row (at most %d of %d blocks computed exactly)" % (k_blk, chosen, VOCAB // 128)
+        if k_blk else " (exact: full logits, slice sorts, merge)"), "rows": ROWS, "resident_GB": round((blob.numel() + (screen if k_blk else 0)) / 1e9, 2)}
+    w.counters_key = None
+    w.cpu = ("exl3_matvec", (blob, bits, u[0].cpu().numpy()))
+    w.keep = (sess, blob, u)
     return w
 
 
@@ -547,6 +579,8 @@ def build_workload(name, torch, sz, synth, synth_device, stream, args):
         return iq3s_prefill(torch, sz, synth, synth_device, stream, args.tokens)
     if name == "exl3head":
         return exl3_head(torch, sz, synth, synth_device, stream, args.bits)
+    if name == "exl3top":
+        return exl3_head_top(torch, sz, synth, synth_device, stream, args.bits, args.screen)
     if name == "stage":
         return stage_exl3_layer(torch, sz, synth, stream)
     return snapshot_states(torch, sz, stream)
@@ -558,10 +592,11 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--layers", type=int, default=48)
-    ap.add_argument("--workload", default="config5", choices=["config1", "config2", "config3", "config4", "config5", "exl3head", "stage", "snapshot"])
+    ap.add_argument("--workload", default="config5", choices=["config1", "config2", "config3", "config4", "config5", "exl3head", "exl3top", "stage", "snapshot"])
     ap.add_argument("--rows", type=int, default=4, help="rows of the verify batch (config3, config5, exl3head; the configurations name 4; 1..8)")
     ap.add_argument("--tokens", type=int, default=512, help="tokens of the prefill chunk (config4 only; the configuration names 512)")
-    ap.add_argument("--bits", type=int, default=4, help="bits a weight of the EXL3 head (exl3head only)")
+    ap.add_argument("--bits", type=int, default=4, help="bits a weight of the EXL3 head (exl3head, exl3top)")
+    ap.add_argument("--screen", type=int, default=0, help="exl3top: blocks a row of the inexact 2-bit screen (0: the exact hand-off)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true", help="default workload only: do not time configurations 1-4 after it")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",

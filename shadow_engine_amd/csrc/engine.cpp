@@ -544,7 +544,7 @@ int head_proxy_sparse(sz_session* s, uint32_t m, uint64_t u, uint32_t need_k, ui
     }
     {
         const sz_arg a[] = {P(s->hp.bmax.ptr), U32(n_ob), U32(k_use), P(s->hp.seen.ptr)};
-        if (launch("proxy_pick_rows", m, 1, 1, 256, 0, stream, a)) return 1;
+        if (launch("proxy_pick_rows", m, 1, 1, 1024, 0, stream, a)) return 1;
     }
     {
         const sz_arg a[] = {P(s->hp.seen.ptr), U32(n_ob), U32(max_sel), P(s->hp.sel.ptr)};
@@ -807,9 +807,9 @@ int32_t sz_head_top(sz_session* s, uint32_t m, uint64_t u, uint32_t* top_host, u
         if (head_proxy_sparse(s, m, u, 64, &max_sel, stream)) return 1;
         const uint32_t nbs = (max_sel * 128 + 4095) / 4096;
         const sz_arg a[] = {P(s->hp.logits.ptr), U32(max_sel * 128), P(s->hp.sel.ptr), U32(nbs), P(s->topv.ptr), P(s->topi.ptr)};
-        if (launch("topk_slices_blks", m * nbs, 1, 1, 256, 0, stream, a)) return 1;
+        if (launch("topk_slices_blks", m * nbs, 1, 1, 1024, 0, stream, a)) return 1;
         const sz_arg b[] = {P(s->topv.ptr), P(s->topi.ptr), U32(nbs), P(s->topo.ptr)};
-        if (launch("topk_merge", m, 1, 1, 256, 0, stream, b)) return 1;
+        if (launch("topk_merge", m, 1, 1, 1024, 0, stream, b)) return 1;
         if (sz_stream_synchronize(stream)) return 1;
         return sz_download(top_host, s->topo.ptr, (uint64_t) m * 128 * 4);
     }
@@ -818,9 +818,9 @@ int32_t sz_head_top(sz_session* s, uint32_t m, uint64_t u, uint32_t* top_host, u
         return 1;
     if (head_logits(s, m, u, s->logits.ptr, stream)) return 1;
     const sz_arg a[] = {P(s->logits.ptr), U32(c.vocab), U32(c.vocab), U32(nb), P(s->topv.ptr), P(s->topi.ptr)};
-    if (launch("topk_slices", m * nb, 1, 1, 256, 0, stream, a)) return 1;
+    if (launch("topk_slices", m * nb, 1, 1, 1024, 0, stream, a)) return 1;
     const sz_arg b[] = {P(s->topv.ptr), P(s->topi.ptr), U32(nb), P(s->topo.ptr)};
-    if (launch("topk_merge", m, 1, 1, 256, 0, stream, b)) return 1;
+    if (launch("topk_merge", m, 1, 1, 1024, 0, stream, b)) return 1;
     if (sz_stream_synchronize(stream)) return 1;
     return sz_download(top_host, s->topo.ptr, (uint64_t) m * 128 * 4);
 }

@@ -177,70 +177,155 @@ extern "C" __global__ void __launch_bounds__(256) route_plan_res_small(const flo
 }
 
 // ---------------------------------------------------------------------------------------------------- exact top-64
-// Bitonic sort of 4096 (value, id) pairs in LDS, value descending then id ascending; a NaN counts as -inf.
-__device__ __forceinline__ bool tk_before(float va, u32 ia, float vb, u32 ib) { return va > vb || (va == vb && ia < ib); }
-
-template <u32 N>
-__device__ __forceinline__ void tk_sort_pow2(float* v, u32* id, u32 tid) {
-    for (u32 size = 2; size <= N; size <<= 1) {
-        for (u32 stride = size >> 1; stride > 0; stride >>= 1) {
-            for (u32 t = tid; t < N / 2; t += 256) {
-                const u32 lo = (t / stride) * 2 * stride + (t % stride), hi = lo + stride;
-                const bool desc = (lo & size) == 0;   // this run sorts best-first
-                const float va = v[lo], vb = v[hi];
-                const u32 ia = id[lo], ib = id[hi];
-                const bool swap = desc ? tk_before(vb, ib, va, ia) : tk_before(va, ia, vb, ib);
-                if (swap) {
-                    v[lo] = vb;
-                    v[hi] = va;
-                    id[lo] = ib;
-                    id[hi] = ia;
-                }
-            }
-            __syncthreads();
-        }
-    }
+// Order (tk_before of the reference, forward.cu:3560): value descending, then id ascending; a NaN counts as -inf, -0 equals +0.
+// A candidate travels as one u64 key that orders exactly like that: the high word is the value's bit pattern made monotonic
+// (-0 folded onto +0), the low word (0x7fffffff - id) * 2 + (1 if the value was -0), and 0 for a slot that holds nothing
+// (value -inf, id 0xffffffff), so value and id come back out of the key bit for bit.
+//
+// A wave keeps its 64 best keys one a lane, sorted; compare-exchange steps are lane exchanges (DPP and lane swaps, no LDS, no
+// barrier): a bitonic sort of 64 keys is 21 steps, and two sorted runs of opposite direction give their 64 best as the
+// lane-wise larger key, a bitonic run that 6 more steps sort.  Which lanes keep the larger key of a step is a compile-time
+// 64-bit constant, so a step is two lane moves, one 64-bit compare, a scalar xor of the compare's mask with the constant, and
+// two selects.  (A 4096-key bitonic sort through LDS with a barrier a step, which this replaces, took 134 us a launch for
+// the slices of four rows of a 151 936-word vocabulary; this takes a tenth.)
+__device__ __forceinline__ u64 tk_key(float x, u32 id) {
+    u32 b = f32_bits(x);
+    if (x != x) b = 0xff800000u;
+    const u32 negz = b == 0x80000000u ? 1u : 0u;
+    if (negz) b = 0u;
+    const u32 o = b ^ ((u32) ((i32) b >> 31) | 0x80000000u);
+    const u32 lo = id == 0xffffffffu ? 0u : ((0x7fffffffu - id) << 1) | negz;
+    return ((u64) o << 32) | lo;
 }
 
-__device__ __forceinline__ void tk_sort4096(float* v, u32* id, u32 tid) { tk_sort_pow2<4096>(v, id, tid); }
+__device__ __forceinline__ void tk_unkey(u64 k, float& x, u32& id) {
+    const u32 o = (u32) (k >> 32), lo = (u32) k;
+    u32 b = (o & 0x80000000u) ? o ^ 0x80000000u : ~o;
+    if (lo & 1u) b = 0x80000000u;
+    x = bits_f32(b);
+    id = lo == 0u ? 0xffffffffu : 0x7fffffffu - (lo >> 1);
+}
+
+#define TK_NOTHING 0x007fffff00000000ull   /* tk_key(-inf, 0xffffffff) */
+
+template <int J>
+__device__ __forceinline__ u64 tk_partner(u64 k, u32 lane) {
+    const u32 lo = f32_bits(lane_xor<J>(bits_f32((u32) k), lane)), hi = f32_bits(lane_xor<J>(bits_f32((u32) (k >> 32)), lane));
+    return ((u64) hi << 32) | lo;
+}
+
+// The lanes that keep the larger key in step (K, J) of a bitonic sort of 64 lanes into descending (DESC) or ascending order:
+// runs of K lanes alternate in direction, the lower lane of a pair J apart keeps the larger key in a descending run.
+template <int K, int J, bool DESC>
+constexpr u64 tk_keep_max() {
+    u64 m = 0;
+    for (int l = 0; l < 64; l++) {
+        const bool main_dir = (l & K) == 0, lower = (l & J) == 0;
+        if (DESC ? main_dir == lower : main_dir != lower) m |= 1ull << l;
+    }
+    return m;
+}
+
+template <int K, int J, bool DESC>
+__device__ __forceinline__ void tk_step(u64& mine, u32 lane) {
+    const u64 other = tk_partner<J>(mine, lane);
+    constexpr u64 keep = tk_keep_max<K, J, DESC>();
+    // where the larger key is kept the partner's is taken unless mine is larger; elsewhere it is taken if mine is larger
+    mine = __builtin_amdgcn_inverse_ballot_w64(__builtin_amdgcn_ballot_w64(mine > other) ^ keep) ? other : mine;
+}
+
+// Bitonic runs of K lanes -> sorted runs of K lanes (K = 64: the whole wave in the order DESC says).
+template <int K, bool DESC>
+__device__ __forceinline__ void tk_merge(u64& v, u32 lane) {
+    if constexpr (K >= 64) tk_step<K, 32, DESC>(v, lane);
+    if constexpr (K >= 32) tk_step<K, 16, DESC>(v, lane);
+    if constexpr (K >= 16) tk_step<K, 8, DESC>(v, lane);
+    if constexpr (K >= 8) tk_step<K, 4, DESC>(v, lane);
+    if constexpr (K >= 4) tk_step<K, 2, DESC>(v, lane);
+    tk_step<K, 1, DESC>(v, lane);
+}
+
+template <bool DESC>
+__device__ __forceinline__ void tk_sort64(u64& v, u32 lane) {
+    tk_merge<2, DESC>(v, lane);
+    tk_merge<4, DESC>(v, lane);
+    tk_merge<8, DESC>(v, lane);
+    tk_merge<16, DESC>(v, lane);
+    tk_merge<32, DESC>(v, lane);
+    tk_merge<64, DESC>(v, lane);
+}
+
+__device__ __forceinline__ u64 tk_larger(u64 a, u64 b) { return a > b ? a : b; }
+
+// best (descending, lane i the i-th best so far) takes in 128 more keys, a and b one a lane each in any order.
+__device__ __forceinline__ void tk_take2(u64& best, u64 a, u64 b, u32 lane) {
+    tk_sort64<false>(a, lane);
+    tk_sort64<true>(b, lane);
+    u64 m = tk_larger(a, b);                 // ascending against descending: the 64 best of the 128, a bitonic run
+    tk_merge<64, false>(m, lane);
+    best = tk_larger(best, m);
+    tk_merge<64, true>(best, lane);
+}
+
+// The 64 best of up to 4096 keys by a workgroup of 4 or 16 waves: key(t) gives key t < n (called with t < 4096 only); 64-key
+// chunks go to the waves in turn, each wave reduces its chunks to 64, and the waves' runs are halved in number through LDS
+// until wave 0 holds the result (descending), which it returns.  sh holds 64 keys a wave.
+template <class F>
+__device__ __forceinline__ u64 tk_best_of_4096(u32 n, F key, u64* sh) {
+    const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+    u64 k[16];
+#pragma unroll
+    for (int c = 0; c < 16; c++) {
+        const u32 t = (c * nw + wave) * 64 + lane;
+        k[c] = (c * nw < 64 && t < n) ? key(t) : TK_NOTHING;
+    }
+    u64 best = TK_NOTHING;
+#pragma unroll
+    for (int c = 0; c < 16; c += 2)
+        if (c * nw < 64 && (c * nw + wave) * 64 < n) tk_take2(best, k[c], k[c + 1], lane);     // uniform over the wave
+    for (u32 half = nw >> 1; half > 0; half >>= 1) {
+        if (wave >= half && wave < 2 * half) sh[wave * 64 + lane] = best;
+        __syncthreads();
+        if (wave < half) {
+            best = tk_larger(best, sh[(wave + half) * 64 + 63 - lane]);     // the other run read backwards: ascending
+            tk_merge<64, true>(best, lane);
+        }
+        __syncthreads();
+    }
+    return best;
+}
 
 // Slice b of row r (blockIdx.x = r * nb + b): the 64 best of logits[r*stride + 4096 b .. +4096) into sv/si[(r*nb + b)*64 ..].
-// Slots past the vocabulary hold (-inf, 0xffffffff).  grid = rows * nb, block 256.
-extern "C" __global__ void __launch_bounds__(256) topk_slices(const float* logits, u32 vocab, u32 stride, u32 nb, float* sv, u32* si) {
-    __shared__ float v[4096];
-    __shared__ u32 id[4096];
-    const u32 tid = threadIdx.x, r = blockIdx.x / nb, b = blockIdx.x % nb;
-    for (u32 t = tid; t < 4096; t += 256) {
-        const u32 i = b * 4096 + t;
-        float x = i < vocab ? logits[(u64) r * stride + i] : -__builtin_inff();
-        if (x != x) x = -__builtin_inff();
-        v[t] = x;
-        id[t] = i < vocab ? i : 0xffffffffu;
-    }
-    __syncthreads();
-    tk_sort4096(v, id, tid);
-    if (tid < 64) {
-        sv[(u64) blockIdx.x * 64 + tid] = v[tid];
-        si[(u64) blockIdx.x * 64 + tid] = id[tid];
+// Slots past the vocabulary hold (-inf, 0xffffffff).  grid = rows * nb, block 1024 (or 256).
+extern "C" __global__ void __launch_bounds__(1024) topk_slices(const float* logits, u32 vocab, u32 stride, u32 nb, float* sv, u32* si) {
+    __shared__ u64 sh[1024];
+    const u32 r = blockIdx.x / nb, b = blockIdx.x % nb;
+    const float* row = logits + (u64) r * stride;
+    const u32 first = b * 4096, n = vocab > first ? min(4096u, vocab - first) : 0u;
+    const u64 best = tk_best_of_4096(n, [&](u32 t) { return tk_key(row[first + t], first + t); }, sh);
+    if (threadIdx.x < 64) {
+        float x;
+        u32 id;
+        tk_unkey(best, x, id);
+        sv[(u64) blockIdx.x * 64 + threadIdx.x] = x;
+        si[(u64) blockIdx.x * 64 + threadIdx.x] = id;
     }
 }
 
 // Row r = blockIdx.x: the 64 best of its nb * 64 slice winners (nb <= 64) into out[r*128 .. +64) (value bits) and
-// out[r*128 + 64 .. +64) (ids).  grid = rows, block 256.
-extern "C" __global__ void __launch_bounds__(256) topk_merge(const float* sv, const u32* si, u32 nb, u32* out) {
-    __shared__ float v[4096];
-    __shared__ u32 id[4096];
-    const u32 tid = threadIdx.x, r = blockIdx.x;
-    for (u32 t = tid; t < 4096; t += 256) {
-        const bool in = t < nb * 64;
-        v[t] = in ? sv[(u64) r * nb * 64 + t] : -__builtin_inff();
-        id[t] = in ? si[(u64) r * nb * 64 + t] : 0xffffffffu;
-    }
-    __syncthreads();
-    tk_sort4096(v, id, tid);
-    if (tid < 64) {
-        out[(u64) r * 128 + tid] = f32_bits(v[tid]);
-        out[(u64) r * 128 + 64 + tid] = id[tid];
+// out[r*128 + 64 .. +64) (ids).  grid = rows, block 1024 (or 256).
+extern "C" __global__ void __launch_bounds__(1024) topk_merge(const float* sv, const u32* si, u32 nb, u32* out) {
+    __shared__ u64 sh[1024];
+    const u32 r = blockIdx.x;
+    const float* v = sv + (u64) r * nb * 64;
+    const u32* id = si + (u64) r * nb * 64;
+    const u64 best = tk_best_of_4096(min(nb * 64, 4096u), [&](u32 t) { return tk_key(v[t], id[t]); }, sh);
+    if (threadIdx.x < 64) {
+        float x;
+        u32 i;
+        tk_unkey(best, x, i);
+        out[(u64) r * 128 + threadIdx.x] = f32_bits(x);
+        out[(u64) r * 128 + 64 + threadIdx.x] = i;
     }
 }
 
@@ -253,14 +338,21 @@ extern "C" __global__ void __launch_bounds__(256) topk_merge(const float* sv, co
 // Block ob = blockIdx.x, lane = output r of the block.  The score of r for row j: over the input blocks b in order,
 // acc = fma(sh, fma(2 x_sc[j][b], sum_i code_i * u_i, x_corr[j][b]), acc) — the integer sums are dot-products-of-four of a
 // code word with four levels (the level word shifted by 2 sl and masked gives inputs 4 sl' ..), exact in any order; the
-// f32 part is the reference's, operation by operation.  The rows' codes are the same for every lane (scalar loads).
+// f32 part is the reference's, operation by operation.  The rows' codes are the same for every lane: they sit in LDS and
+// are read as broadcasts, four words at a time.
 // bmax[j * n_ob + ob] = the largest score of the block.  grid = out / 128, block 128.
 template <int M>
 __device__ __forceinline__ void proxy_q2_bmax(const u32* __restrict__ w_q2, const u16* __restrict__ w_sc, const u32* __restrict__ xq,
                                               const float* __restrict__ x_sc, const float* __restrict__ x_corr, float* __restrict__ bmax,
                                               u32 n_ob, u32 in_f, u32 m) {
+    __shared__ __attribute__((aligned(16))) u32 s_xq[M][1024];      // the rows' codes: in <= 4096
     __shared__ float s_mx[2][M];
     const u32 ob = blockIdx.x, r = threadIdx.x, n_b = in_f / 128;
+    for (u32 i = r; i < M * n_b * 32; i += 128) {
+        const u32 j = i / (n_b * 32), k = i % (n_b * 32);
+        s_xq[j][k] = j < m ? xq[(u64) j * n_b * 32 + k] : 0u;
+    }
+    __syncthreads();
     const u32x4* wq = (const u32x4*) w_q2 + (u64) ob * n_b * 256 + r;
     const u16* sc = w_sc + (u64) ob * n_b * 128 + r;
     float acc[M];
@@ -276,14 +368,17 @@ __device__ __forceinline__ void proxy_q2_bmax(const u32* __restrict__ w_q2, cons
 #pragma unroll
         for (int hb = 0; hb < 2; hb++)
 #pragma unroll
-            for (int wi = 0; wi < 4; wi++)
+            for (int wi = 0; wi < 4; wi++) {
+                u32 u[4];
 #pragma unroll
-                for (int sl = 0; sl < 4; sl++) {
-                    const u32 u = (q[hb][wi] >> (2 * sl)) & 0x03030303u;
+                for (int sl = 0; sl < 4; sl++) u[sl] = (q[hb][wi] >> (2 * sl)) & 0x03030303u;
 #pragma unroll
-                    for (int j = 0; j < M; j++)
-                        ia[j] = __builtin_amdgcn_sdot4((i32) xq[((u64) min((u32) j, m - 1) * n_b + b) * 32 + hb * 16 + wi * 4 + sl], (i32) u, ia[j], false);
+                for (int j = 0; j < M; j++) {
+                    const u32x4 xv = *(const u32x4*) &s_xq[j][b * 32 + hb * 16 + wi * 4];      // the same address in every lane
+#pragma unroll
+                    for (int sl = 0; sl < 4; sl++) ia[j] = __builtin_amdgcn_sdot4((i32) xv[sl], (i32) u[sl], ia[j], false);
                 }
+            }
 #pragma unroll
         for (int j = 0; j < M; j++) {
             const u64 at = (u64) min((u32) j, m - 1) * n_b + b;
@@ -313,45 +408,60 @@ extern "C" __global__ void __launch_bounds__(128) proxy_q2_bmax_m8(const u32* w_
 }
 
 // Row j = blockIdx.x: marks the k_blk best blocks of bmax[j][0 .. n_ob) in the bit map `seen` (forward.cu:4519-4563, with its
-// way of choosing: thread t keeps the four best of blocks t, t + 256, .. — a strictly larger value replaces the fourth, so of
-// equal values the earlier block stays; a NaN counts as -3e38 — and the 1024 kept are ordered by value descending, block
-// ascending; a thread that holds five of the k_blk best loses one, as there).  grid = m, block 256.
-extern "C" __global__ void __launch_bounds__(256) proxy_pick_rows(const float* bmax, u32 n_ob, u32 k_blk, u32* seen) {
-    __shared__ float v[1024];
-    __shared__ u32 id[1024];
-    const u32 tid = threadIdx.x;
+// way of choosing: thread t < 256 keeps the four best of blocks t, t + 256, .. — a strictly larger value replaces the fourth,
+// so of equal values the earlier block stays; a NaN counts as -3e38 — and of the 1024 kept, ordered by value descending, block
+// ascending, the first k_blk are marked; a thread that holds five of the k_blk best loses one, as there).  Only the set matters,
+// so nothing is sorted across waves: each of the 16 waves sorts its 64 candidates and a candidate's place in the whole order
+// is its place in its own run plus, by binary search, the number of better keys in the other 15.  grid = m, block 1024.
+extern "C" __global__ void __launch_bounds__(1024) proxy_pick_rows(const float* bmax, u32 n_ob, u32 k_blk, u32* seen) {
+    __shared__ u64 cand[1024];
+    const u32 tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const float* row = bmax + (u64) blockIdx.x * n_ob;
-    float lv[4] = {-3.0e38f, -3.0e38f, -3.0e38f, -3.0e38f};
-    u32 li[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
-    for (u32 i = tid; i < n_ob; i += 256) {
-        float x = row[i];
-        if (x != x) x = -3.0e38f;
-        if (x > lv[3]) {
-            lv[3] = x;
-            li[3] = i;
+    if (tid < 256) {
+        float lv[4] = {-3.0e38f, -3.0e38f, -3.0e38f, -3.0e38f};
+        u32 li[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+        for (u32 i = tid; i < n_ob; i += 256) {
+            float x = row[i];
+            if (x != x) x = -3.0e38f;
+            if (x > lv[3]) {
+                lv[3] = x;
+                li[3] = i;
 #pragma unroll
-            for (int k = 3; k > 0; k--)
-                if (tk_before(lv[k], li[k], lv[k - 1], li[k - 1])) {
-                    const float tv = lv[k];
-                    lv[k] = lv[k - 1];
-                    lv[k - 1] = tv;
-                    const u32 ti = li[k];
-                    li[k] = li[k - 1];
-                    li[k - 1] = ti;
-                }
+                for (int k = 3; k > 0; k--)
+                    if (lv[k] > lv[k - 1] || (lv[k] == lv[k - 1] && li[k] < li[k - 1])) {
+                        const float tv = lv[k];
+                        lv[k] = lv[k - 1];
+                        lv[k - 1] = tv;
+                        const u32 ti = li[k];
+                        li[k] = li[k - 1];
+                        li[k - 1] = ti;
+                    }
+            }
         }
-    }
 #pragma unroll
-    for (int k = 0; k < 4; k++) {
-        v[tid * 4 + k] = lv[k];
-        id[tid * 4 + k] = li[k];
+        for (int k = 0; k < 4; k++) cand[tid * 4 + k] = tk_key(lv[k], li[k]);
     }
     __syncthreads();
-    tk_sort_pow2<1024>(v, id, tid);
-    for (u32 t = tid; t < k_blk && t < n_ob && t < 1024; t += 256) {
-        const u32 ob = id[t];
-        if (ob < n_ob) atomicOr(&seen[ob >> 5], 1u << (ob & 31));
+    u64 mine = cand[tid];
+    tk_sort64<true>(mine, lane);
+    __syncthreads();
+    cand[tid] = mine;
+    __syncthreads();
+    u32 rank = lane;
+#pragma unroll
+    for (u32 w = 0; w < 16; w++) {
+        const u64* run = cand + w * 64;       // descending
+        u32 c = 0;                            // keys of the run that are better than mine
+#pragma unroll
+        for (u32 step = 32; step > 0; step >>= 1)
+            if (run[c + step - 1] > mine) c += step;
+        if (run[c] > mine) c++;
+        if (w != wave) rank += c;
     }
+    float x;
+    u32 ob;
+    tk_unkey(mine, x, ob);
+    if (rank < k_blk && rank < n_ob && ob < n_ob) atomicOr(&seen[ob >> 5], 1u << (ob & 31));
 }
 
 // The marked blocks in ascending order into sel[1 ..], their number (at most max_sel; what does not fit is dropped) into
@@ -384,25 +494,21 @@ extern "C" __global__ void __launch_bounds__(64) proxy_compact_seen(u32* seen, u
 }
 
 // topk_slices over the packed logits of a block list (forward.cu:4626-4647): element i of row r (i < 128 sel[0]) is output
-// sel[1 + i / 128] * 128 + i % 128; elements past the list hold (-inf, 0xffffffff).  Since the list ascends, packed order is
-// output order and ties go to the lower output as everywhere.  grid = rows * nb, block 256.
-extern "C" __global__ void __launch_bounds__(256) topk_slices_blks(const float* logits, u32 stride, const u32* sel, u32 nb, float* sv, u32* si) {
-    __shared__ float v[4096];
-    __shared__ u32 id[4096];
-    const u32 tid = threadIdx.x, r = blockIdx.x / nb, b = blockIdx.x % nb;
-    const u32 n = sel[0] << 7;
-    for (u32 t = tid; t < 4096; t += 256) {
-        const u32 i = b * 4096 + t;
-        float x = i < n ? logits[(u64) r * stride + i] : -__builtin_inff();
-        if (x != x) x = -__builtin_inff();
-        v[t] = x;
-        id[t] = i < n ? (sel[1 + (i >> 7)] << 7) | (i & 127) : 0xffffffffu;
-    }
-    __syncthreads();
-    tk_sort4096(v, id, tid);
-    if (tid < 64) {
-        sv[(u64) blockIdx.x * 64 + tid] = v[tid];
-        si[(u64) blockIdx.x * 64 + tid] = id[tid];
+// sel[1 + i / 128] * 128 + i % 128; elements past the list hold (-inf, 0xffffffff).  The list ascends, so packed order is
+// output order: candidates are ordered by their place and the place is turned into the output at the end.  grid = rows * nb,
+// block 1024 (or 256).
+extern "C" __global__ void __launch_bounds__(1024) topk_slices_blks(const float* logits, u32 stride, const u32* sel, u32 nb, float* sv, u32* si) {
+    __shared__ u64 sh[1024];
+    const u32 r = blockIdx.x / nb, b = blockIdx.x % nb;
+    const float* row = logits + (u64) r * stride;
+    const u32 total = sel[0] << 7, first = b * 4096, n = total > first ? min(4096u, total - first) : 0u;
+    const u64 best = tk_best_of_4096(n, [&](u32 t) { return tk_key(row[first + t], first + t); }, sh);
+    if (threadIdx.x < 64) {
+        float x;
+        u32 at;
+        tk_unkey(best, x, at);
+        sv[(u64) blockIdx.x * 64 + threadIdx.x] = x;
+        si[(u64) blockIdx.x * 64 + threadIdx.x] = at == 0xffffffffu ? at : (sel[1 + (at >> 7)] << 7) | (at & 127);
     }
 }
 

@@ -864,8 +864,9 @@ def test_head_argmax_prefers_the_lowest_id_on_exact_ties(gpu):
     assert int(ids[0]) == min([best] + others)
 
 
-def test_top64_on_adversarial_rows(gpu):
-    # crates/shadowzero-cuda/tests/topk.rs: ties, all equal, -inf and NaN, winners in the ragged last slice
+@pytest.mark.parametrize("block", [256, 1024])
+def test_top64_on_adversarial_rows(gpu, block):
+    # crates/shadowzero-cuda/tests/topk.rs: ties, all equal, -inf and NaN, winners in the ragged last slice; and zeros of both signs
     rng = np.random.default_rng(14)
     vocab = 151936
     u = rng.random((5, vocab)).astype(np.float32)
@@ -878,15 +879,18 @@ def test_top64_on_adversarial_rows(gpu):
     rows[3, 12345] = np.nan
     rows[4] = u[4]
     rows[4, vocab - 100:] += 50
+    rows[2, 5::7] = -1.25                                     # two values only, so the 64 are the lowest ids of the larger
+    rows[1] -= 19.5                                           # steps of 0.5 up to zero, and zeros of both signs at the top:
+    rows[1, 3::11] = -0.0                                     # -0 equals +0, the order among them is by id, the sign comes back as it was
     nb = (vocab + 4095) // 4096
     dl = dev(gpu, rows)
     sv = gpu.empty(5 * nb * 64, dtype=gpu.float32, device="cuda")
     si = gpu.empty(5 * nb * 64, dtype=gpu.int32, device="cuda")
     out = gpu.empty(5 * 128, dtype=gpu.int32, device="cuda")
     A = sz.Arg
-    sz.launch("topk_slices", (5 * nb, 1, 1), (256, 1, 1), 0, 0,
+    sz.launch("topk_slices", (5 * nb, 1, 1), (block, 1, 1), 0, 0,
               [A.ptr(dl.data_ptr()), A.u32(vocab), A.u32(vocab), A.u32(nb), A.ptr(sv.data_ptr()), A.ptr(si.data_ptr())])
-    sz.launch("topk_merge", (5, 1, 1), (256, 1, 1), 0, 0, [A.ptr(sv.data_ptr()), A.ptr(si.data_ptr()), A.u32(nb), A.ptr(out.data_ptr())])
+    sz.launch("topk_merge", (5, 1, 1), (block, 1, 1), 0, 0, [A.ptr(sv.data_ptr()), A.ptr(si.data_ptr()), A.u32(nb), A.ptr(out.data_ptr())])
     gpu.cuda.synchronize()
     words = out.cpu().numpy().view(np.uint32).reshape(5, 128)
     for r in range(5):

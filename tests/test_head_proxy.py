@@ -356,7 +356,7 @@ def test_the_reference_test_through_the_kernels(gpu):
     sz.launch("head_exl3_5", (n_ob, 1, 1), (256, 1, 1), lds, 0, [P(db), P(xa), P(inv), P(dense), A.u32(rows), P(part), A.u32(cols), A.u32(rows), A.u32(m), A.ptr(0)])
     sz.launch("proxy_q2_quant_x", (n_b, m, 1), (64, 1, 1), 0, 0, [P(db), P(dx), A.u32(cols), P(xq), P(xsc), P(xcorr), A.u32(cols)])
     sz.launch("proxy_q2_bmax_m4", (n_ob, 1, 1), (128, 1, 1), 0, 0, [P(wq), P(ws), P(xq), P(xsc), P(xcorr), P(bmax), A.u32(n_ob), A.u32(cols), A.u32(m)])
-    sz.launch("proxy_pick_rows", (m, 1, 1), (256, 1, 1), 0, 0, [P(bmax), A.u32(n_ob), A.u32(k_blk), P(seen)])
+    sz.launch("proxy_pick_rows", (m, 1, 1), (1024, 1, 1), 0, 0, [P(bmax), A.u32(n_ob), A.u32(k_blk), P(seen)])
     sz.launch("proxy_compact_seen", (1, 1, 1), (64, 1, 1), 0, 0, [P(seen), A.u32(n_ob), A.u32(max_sel), P(sel)])
     sz.launch("head_exl3_5", (max_sel, 1, 1), (256, 1, 1), lds, 0, [P(db), P(xa), P(inv), P(sparse), A.u32(max_sel * 128), P(part), A.u32(cols), A.u32(rows), A.u32(m), P(sel)])
     sz.launch("topk_slices_blks", (m * nbs, 1, 1), (256, 1, 1), 0, 0, [P(sparse), A.u32(max_sel * 128), P(sel), A.u32(nbs), P(sv), P(si)])
