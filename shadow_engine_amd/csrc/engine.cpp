@@ -573,6 +573,7 @@ int head_argmax(sz_session* s, uint32_t m, uint64_t u, uint64_t ids, uint64_t st
 int head_logits(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uint64_t stream) {
     if (head_check(s, m, u, "sz_head_logits")) return 1;
     if (head_is_exl3(s)) return head_exl3(s, m, u, logits, 0, stream);
+    if (head_mfma_ok(s)) return head_argmax_mfma(s, m, u, logits, s->ids.ptr, stream);   // one pass for all rows; the ids are a by-product
     const sz_session_config& c = s->cfg;
     return matvec_cols_dev(s->head_type, s->head_w, c.hidden, c.vocab, u, c.hidden, logits, c.vocab, m, 0, 0, stream);
 }
