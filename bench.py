@@ -279,7 +279,7 @@ def exl3_head_top(torch, sz, synth, synth_device, stream, bits, k_blk):
     w.describe = {"workload": "top-64 hand-off of the EXL3 lm_head 151936 x 2048 at K = %d for %d rows, to the host%s" % (
         bits, ROWS, " through the inexact 2-bit screen, %d blocks a row (at most %d of %d blocks computed exactly)" % (k_blk, chosen, VOCAB // 128)
         if k_blk else " (exact: full logits, slice sorts, merge)"), "rows": ROWS, "resident_GB": round((blob.numel() + (screen if k_blk else 0)) / 1e9, 2)}
-    w.counters_key = None
+    w.counters_key = {0: "exl3top", 128: "exl3top_screen"}.get(k_blk) if (bits == 4 and ROWS == 4) else None
     w.cpu = ("exl3_matvec", (blob, bits, u[0].cpu().numpy()))
     w.keep = (sess, blob, u)
     return w

@@ -231,7 +231,12 @@ __device__ __forceinline__ void tk_step(u64& mine, u32 lane) {
     const u64 other = tk_partner<J>(mine, lane);
     constexpr u64 keep = tk_keep_max<K, J, DESC>();
     // where the larger key is kept the partner's is taken unless mine is larger; elsewhere it is taken if mine is larger
-    mine = __builtin_amdgcn_inverse_ballot_w64(__builtin_amdgcn_ballot_w64(mine > other) ^ keep) ? other : mine;
+    const u64 take = __builtin_amdgcn_ballot_w64(mine > other) ^ keep;
+#if __has_builtin(__builtin_amdgcn_inverse_ballot_w64)
+    mine = __builtin_amdgcn_inverse_ballot_w64(take) ? other : mine;     // the mask selects as it stands: no vector work
+#else
+    mine = ((take >> lane) & 1) ? other : mine;                          // a compiler without it (an older run-time compiler) shifts
+#endif
 }
 
 // Bitonic runs of K lanes -> sorted runs of K lanes (K = 64: the whole wave in the order DESC says).

@@ -28,13 +28,16 @@ import sqlite3
 import sys
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-OURS = ("verify_", "decode_", "head_", "argmax_merge", "copy_", "matvec_", "route_", "swiglu", "moe_", "prefill_", "quant_act", "scatter_", "exl3_", "topk_")
+OURS = ("verify_", "decode_", "head_", "argmax_merge", "copy_", "matvec_", "route_", "swiglu", "moe_", "prefill_", "quant_act", "scatter_", "exl3_", "topk_", "proxy_")
 NAMES = {"config5": ("verify_round_config5", "the default benchmark workload (config 5: 48-layer verify round on a 4-row batch, mixed EXL3 K in {2,3,4}, Q8_0 lm_head)", ""),
          "config3": ("verify_layer_and_head_config3", "bench.py --workload config3 (one EXL3 K=3 MoE layer for 4 tokens + Q8_0 head + acceptance)", " --workload config3"),
          "config1": ("matvec_q8_0_config1", "bench.py --workload config1 (one Q8_0 1024 x 2048 matrix-vector product)", " --workload config1"),
          "config2": ("iq3s_decode_layer_config2", "bench.py --workload config2 (IQ3_S MoE layer for one token, 8 different layers a step)", " --workload config2"),
          "config4": ("prefill_chunk_config4", "bench.py --workload config4 (prefill chunk: 512 tokens through 512 IQ3_S experts, int8 matrix cores)", " --workload config4"),
          "exl3head": ("head_exl3_k4_lm_head", "bench.py --workload exl3head (EXL3 K=4 lm_head 151936 x 2048, 4-row batch, arg-max fused in)", " --workload exl3head"),
+         "exl3top": ("head_exl3_k4_top64", "bench.py --workload exl3top (top-64 hand-off of the EXL3 K=4 lm_head 151936 x 2048 for 4 rows, exact)", " --workload exl3top"),
+         "exl3top_screen": ("head_exl3_k4_top64_screened", "bench.py --workload exl3top --screen 128 (the same hand-off through the inexact 2-bit screen, 128 blocks a row)",
+                            " --workload exl3top --screen 128"),
          "stage": ("stage_exl3_layer", "bench.py --workload stage (one EXL3 layer of a safetensors checkpoint staged into HBM)", " --workload stage"),
          "snapshot": ("copy_ranges_snapshot", "bench.py --workload snapshot (73 device ranges saved and put back)", " --workload snapshot")}
 SQ1 = "SQ_INSTS_VALU SQ_ACTIVE_INST_VALU SQ_BUSY_CYCLES SQ_WAVES SQ_WAVE_CYCLES SQ_WAIT_INST_ANY SQ_INSTS_SALU SQ_INSTS_LDS"
