@@ -29,6 +29,14 @@ def test_library_exports_every_declared_symbol():
     assert set(names) == set(sz.exported_symbols()), "the Python binding and the header list different entry points"
 
 
+def test_header_is_plain_c():
+    """The boundary is a C ABI: the header must compile as C99 (what a cgo / bindgen / ctypes user feeds it to) and as C++."""
+    import subprocess
+    h = os.path.join(ROOT, "include", "shadowzero_hip.h")
+    subprocess.run(["gcc", "-std=c99", "-Wall", "-Wextra", "-Werror", "-pedantic", "-fsyntax-only", "-x", "c", h], check=True)
+    subprocess.run(["g++", "-std=c++17", "-Wall", "-Werror", "-fsyntax-only", "-x", "c++", h], check=True)
+
+
 def test_registry_matches_the_kernel_sources():
     want = [(name, build.FILES[fi][0], kinds) for name, fi, kinds in build.registry_entries()]
     kind_id = {"SZ_P_PTR": 0, "SZ_P_CONSTPTR": 1, "SZ_P_U32": 2, "SZ_P_I32": 3, "SZ_P_U64": 4, "SZ_P_F32": 5}
@@ -38,7 +46,8 @@ def test_registry_matches_the_kernel_sources():
     names = [n for n, _, _ in got]
     assert len(names) == len(set(names))
     for expected in ("matvec_q8_0", "matvec_cols_iq3_s", "matvec_grouped_exl3_3", "exl3_decode_8", "route_plan_res_small",
-                     "moe_combine_qwen_rows", "head_q8_0_argmax", "topk_merge", "verify_accept"):
+                     "moe_combine_qwen_rows", "head_q8_0_argmax", "topk_merge", "verify_accept", "exl3_build_q2_proxy_5",
+                     "proxy_q2_bmax_m4", "proxy_pick_rows", "topk_slices_blks"):
         assert expected in names
 
 
