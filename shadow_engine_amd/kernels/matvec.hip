@@ -145,6 +145,14 @@ __device__ __forceinline__ void unit_dot_q8_0(u32 o, u32 u, const float (&x)[32]
 
 __shared__ u32 sz_iq3s_grid[512];
 
+// The signs of four weights (bits 0..3 of n) applied to their packed magnitudes (four bytes, each at most 15): a set bit
+// negates its byte.  n * 0x00204081 puts bit i of n at bit 8 i (and others in between), the mask leaves 0 or 1 a byte, times 255 is
+// 0x00 or 0xff a byte, and (m ^ ff) + 1 = -m byte by byte (no carries: the magnitudes are below 128, and -m + ... stays in its byte).
+__device__ __forceinline__ u32 iq3s_signed4(u32 mags, u32 n) {
+    const u32 one = (n * 0x00204081u) & 0x01010101u;
+    return (mags ^ (one * 255u)) + one;
+}
+
 template <int M>
 __device__ __forceinline__ void unit_dot_iq3_s(u32 o, u32 u, const float (&x)[32][M], float (&out)[M]) {
     const u32 b = o + 110 * (u >> 3), g = u & 7;
@@ -161,13 +169,14 @@ __device__ __forceinline__ void unit_dot_iq3_s(u32 o, u32 u, const float (&x)[32
     for (int j = 0; j < M; j++) acc[j] = 0.0f;
 #pragma unroll
     for (int jj = 0; jj < 8; jj++) {
-        const u32 q = ((jj < 4 ? qs0 : qs1) >> (8 * (jj & 3))) & 0xff;
-        const u32 grid = sz_iq3s_grid[q | (((qh >> jj) & 1u) << 8)];
+        // the table's byte offset: 4 * (index byte | high bit << 8), from two bit-field extracts, a shift and a shift-or
+        const u32 at = (__builtin_amdgcn_ubfe(jj < 4 ? qs0 : qs1, 8 * (jj & 3), 8) << 2) | (__builtin_amdgcn_ubfe(qh, jj, 1) << 10);
+        const u32 grid = *(const u32*) ((const u8*) sz_iq3s_grid + at);
+        const u32 sg = iq3s_signed4(grid, __builtin_amdgcn_ubfe(signs, 4 * jj, 4));
 #pragma unroll
         for (int k = 0; k < 4; k++) {
             const int i = 4 * jj + k;
-            const float mag = (float) ((grid >> (8 * k)) & 0xff);
-            const float w = bits_f32(f32_bits(mag) | ((signs << (31 - i)) & 0x80000000u));
+            const float w = (float) (i8) (sg >> (8 * k));        // one sign-extending byte conversion
 #pragma unroll
             for (int j = 0; j < M; j++) acc[j] = __builtin_fmaf(w, x[i][j], acc[j]);
         }
