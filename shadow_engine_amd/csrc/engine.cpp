@@ -294,7 +294,7 @@ struct sz_session {
     int head_type = 0;
     uint64_t head_w = 0;
     // batch buffers (session.rs `bb`): the plan, the expert products, the split-k partials, the head's scratch
-    DevBuf plan, eg, act, eo, part, dn, head_part, logits, topv, topi, topo, ids;
+    DevBuf plan, eg, act, eo, part, dn, head_part, logits, topv, topi, ids;
     DevBuf head_xa, head_inv;   // an EXL3 head's rotated inputs as f16 high and low parts (16 rows of 128 a 128-block), and the tokens' scales
     DevBuf rl, sgl;   // the router's outputs for a batch: f32[max_rows][n_expert], f32[max_rows]
     // the optional 2-bit screen of an EXL3 head (HeadProxy of session.rs:428-441): k_blk = 0 is off
@@ -305,6 +305,7 @@ struct sz_session {
     struct {
         DevBuf xq, xd, tidx, w, cnt, offs, list, items, hq, hd, eo;
     } pf;   // the prefill chunk's buffers, grown on demand
+    void* top_host = nullptr;  // pinned host memory the top-64 merge writes to directly (8 rows of 128 words): no copy back
     bool last_fused = false;   // the last layer call left its routing in the fused layout [tidx | w | cnt]
     std::map<SzGraphKey, uint64_t> graphs;
     // plan offsets for the largest batch
@@ -612,6 +613,7 @@ sz_session* sz_session_new(const sz_session_config* cfg) {
 
 void sz_session_free(sz_session* s) {
     if (!s) return;
+    if (s->top_host) hip().hipHostFree(s->top_host);
     for (auto& g : s->graphs) sz_graph_destroy(g.second);
     delete s;
 }
@@ -795,35 +797,43 @@ int32_t sz_head_logits(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, u
     return head_logits(s, m, u, logits, stream);
 }
 
+// The merge kernel's output goes straight into pinned host memory (device-visible, coherent): once the stream has drained the
+// 2 KiB a row are there, and no copy from device memory (a blocking driver call of its own) is needed.
+static int top_finish(sz_session* s, uint32_t m, uint32_t* top_host, uint64_t stream) {
+    if (sz_stream_synchronize(stream)) return 1;
+    std::memcpy(top_host, s->top_host, (size_t) m * 128 * 4);
+    return 0;
+}
+
 int32_t sz_head_top(sz_session* s, uint32_t m, uint64_t u, uint32_t* top_host, uint64_t stream) {
     clear_error();
     if (!s) return fail("sz_head_top: null session");
+    if (!s->top_host && hip_check(hip().hipHostMalloc(&s->top_host, 8 * 128 * 4, 0), "hipHostMalloc")) return 1;
+    const uint64_t topo = (uint64_t) s->top_host;
     const sz_session_config& c = s->cfg;
     const uint32_t nb = (c.vocab + 4095) / 4096;
     if (nb > 64) return fail("sz_head_top: vocabulary above 262144");
     if (head_check(s, m, u, "sz_head_top")) return 1;
     if (s->hp.k_blk) {   // head_top_at, session.rs:5997-6022: the screened form, the top 64 among the chosen blocks
-        if (s->topv.need(8ull * 64 * 64 * 4) || s->topi.need(8ull * 64 * 64 * 4) || s->topo.need(8ull * 128 * 4)) return 1;
+        if (s->topv.need(8ull * 64 * 64 * 4) || s->topi.need(8ull * 64 * 64 * 4)) return 1;
         uint32_t max_sel = 0;
         if (head_proxy_sparse(s, m, u, 64, &max_sel, stream)) return 1;
         const uint32_t nbs = (max_sel * 128 + 4095) / 4096;
         const sz_arg a[] = {P(s->hp.logits.ptr), U32(max_sel * 128), P(s->hp.sel.ptr), U32(nbs), P(s->topv.ptr), P(s->topi.ptr)};
         if (launch("topk_slices_blks", m * nbs, 1, 1, 1024, 0, stream, a)) return 1;
-        const sz_arg b[] = {P(s->topv.ptr), P(s->topi.ptr), U32(nbs), P(s->topo.ptr)};
+        const sz_arg b[] = {P(s->topv.ptr), P(s->topi.ptr), U32(nbs), P(topo)};
         if (launch("topk_merge", m, 1, 1, 1024, 0, stream, b)) return 1;
-        if (sz_stream_synchronize(stream)) return 1;
-        return sz_download(top_host, s->topo.ptr, (uint64_t) m * 128 * 4);
+        return top_finish(s, m, top_host, stream);
     }
     if (s->logits.need((uint64_t) c.max_rows * c.vocab * 4) || s->topv.need((uint64_t) c.max_rows * nb * 64 * 4) ||
-        s->topi.need((uint64_t) c.max_rows * nb * 64 * 4) || s->topo.need((uint64_t) c.max_rows * 128 * 4))
+        s->topi.need((uint64_t) c.max_rows * nb * 64 * 4))
         return 1;
     if (head_logits(s, m, u, s->logits.ptr, stream)) return 1;
     const sz_arg a[] = {P(s->logits.ptr), U32(c.vocab), U32(c.vocab), U32(nb), P(s->topv.ptr), P(s->topi.ptr)};
     if (launch("topk_slices", m * nb, 1, 1, 1024, 0, stream, a)) return 1;
-    const sz_arg b[] = {P(s->topv.ptr), P(s->topi.ptr), U32(nb), P(s->topo.ptr)};
+    const sz_arg b[] = {P(s->topv.ptr), P(s->topi.ptr), U32(nb), P(topo)};
     if (launch("topk_merge", m, 1, 1, 1024, 0, stream, b)) return 1;
-    if (sz_stream_synchronize(stream)) return 1;
-    return sz_download(top_host, s->topo.ptr, (uint64_t) m * 128 * 4);
+    return top_finish(s, m, top_host, stream);
 }
 
 int32_t sz_verify_accept(const uint32_t* ids, const uint32_t* drafts, uint32_t n_drafts, uint32_t* keep) {
