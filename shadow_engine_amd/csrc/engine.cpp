@@ -164,10 +164,29 @@ int matvec_cols_dev(int ty, uint64_t w, uint64_t cols, uint64_t rows, uint64_t x
 using namespace sz;
 
 // ---- B1: Backend ----------------------------------------------------------------------------------------------------
+// Pinned host memory that the device reads and writes directly (grown on demand, freed with its owner).
+struct PinnedBuf {
+    void* ptr = nullptr;
+    uint64_t bytes = 0;
+    int need(uint64_t n) {
+        if (bytes >= n) return 0;
+        if (ptr) hip().hipHostFree(ptr);
+        ptr = nullptr;
+        bytes = 0;
+        if (hip_check(hip().hipHostMalloc(&ptr, n, 0), "hipHostMalloc")) return 1;
+        bytes = n;
+        return 0;
+    }
+    ~PinnedBuf() {
+        if (ptr) hip().hipHostFree(ptr);
+    }
+};
+
 struct sz_backend {
     uint64_t budget = 0, resident_bytes = 0, uploads = 0;
     std::unordered_map<std::string, DevBuf> resident;
-    DevBuf w, x, y, scratch;
+    DevBuf w, x, scratch;
+    PinnedBuf hx, hy;   // the call's input on its way to the device, and its output, which the kernel writes here itself
 };
 
 extern "C" {
@@ -216,11 +235,17 @@ int32_t sz_matvec(sz_backend* b, int32_t ty, uint64_t cols, uint64_t rows, const
         b->uploads++;
         wp = b->w.ptr;
     }
-    if (b->x.need(cols * 4) || b->y.need(rows * 4) || sz_upload(b->x.ptr, x, cols * 4)) return 1;
+    // x goes through pinned memory with an asynchronous copy and y is written into pinned memory by the kernel itself: the call
+    // waits once, for the stream, instead of once a blocking copy each way (31 -> 20 us a call for a resident 1024 x 2048 matrix)
+    if (b->x.need(cols * 4) || b->hx.need(cols * 4) || b->hy.need(rows * 4)) return 1;
+    std::memcpy(b->hx.ptr, x, cols * 4);
+    if (hip_check(hip().hipMemcpyHtoDAsync((void*) b->x.ptr, b->hx.ptr, cols * 4, nullptr), "hipMemcpyHtoDAsync")) return 1;
     const uint64_t sb = cols_scratch_bytes(f, cols, rows, 1);
     if (sb && b->scratch.need(sb)) return 1;
-    if (matvec_cols_dev(ty, wp, cols, rows, b->x.ptr, (uint32_t) cols, b->y.ptr, (uint32_t) rows, 1, b->scratch.ptr, b->scratch.bytes, 0)) return 1;
-    return sz_download(y, b->y.ptr, rows * 4);   // synchronous: waits for the kernels
+    if (matvec_cols_dev(ty, wp, cols, rows, b->x.ptr, (uint32_t) cols, (uint64_t) b->hy.ptr, (uint32_t) rows, 1, b->scratch.ptr, b->scratch.bytes, 0)) return 1;
+    if (sz_stream_synchronize(0)) return 1;   // synchronous, as the reference's backend: waits for the kernels
+    std::memcpy(y, b->hy.ptr, rows * 4);
+    return 0;
 }
 
 // ---- B4: device entry points ------------------------------------------------------------------------------------------
