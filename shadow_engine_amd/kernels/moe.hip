@@ -262,32 +262,39 @@ __device__ __forceinline__ void tk_sort64(u64& v, u32 lane) {
 
 __device__ __forceinline__ u64 tk_larger(u64 a, u64 b) { return a > b ? a : b; }
 
-// best (descending, lane i the i-th best so far) takes in 128 more keys, a and b one a lane each in any order.
-__device__ __forceinline__ void tk_take2(u64& best, u64 a, u64 b, u32 lane) {
-    tk_sort64<false>(a, lane);
-    tk_sort64<true>(b, lane);
-    u64 m = tk_larger(a, b);                 // ascending against descending: the 64 best of the 128, a bitonic run
-    tk_merge<64, false>(m, lane);
-    best = tk_larger(best, m);
-    tk_merge<64, true>(best, lane);
-}
-
-// The 64 best of up to 4096 keys by a workgroup of 4 or 16 waves: key(t) gives key t < n (called with t < 4096 only); 64-key
-// chunks go to the waves in turn, each wave reduces its chunks to 64, and the waves' runs are halved in number through LDS
-// until wave 0 holds the result (descending), which it returns.  sh holds 64 keys a wave.
-template <class F>
-__device__ __forceinline__ u64 tk_best_of_4096(u32 n, F key, u64* sh) {
+// The 64 best of up to 64 MAXCH keys by a workgroup of nw waves (a power of two; nw * PERW >= MAXCH): key(t) gives key t < n;
+// 64-key chunks go to the waves in turn.  A wave sorts its chunks, alternately ascending and descending — independent
+// chains of lane exchanges that fill each other's issue gaps — and halves their number level by level: the lane-wise larger
+// key of an ascending and a descending run is a bitonic run of the 64 best of both, which 6 steps sort again.  The waves'
+// runs are then halved in number through LDS until wave 0 holds the result (descending), which it returns.  sh holds 64
+// keys a wave.
+template <int MAXCH, int PERW, class F>
+__device__ __forceinline__ u64 tk_best_of(u32 n, F key, u64* sh) {
+    static_assert(PERW >= 2 && (PERW & (PERW - 1)) == 0, "a power of two");
     const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63, nw = blockDim.x >> 6;
-    u64 k[16];
+    u64 k[PERW];
 #pragma unroll
-    for (int c = 0; c < 16; c++) {
+    for (int c = 0; c < PERW; c++) {
         const u32 t = (c * nw + wave) * 64 + lane;
-        k[c] = (c * nw < 64 && t < n) ? key(t) : TK_NOTHING;
+        k[c] = (c * nw < (u32) MAXCH && t < n) ? key(t) : TK_NOTHING;
     }
-    u64 best = TK_NOTHING;
 #pragma unroll
-    for (int c = 0; c < 16; c += 2)
-        if (c * nw < 64 && (c * nw + wave) * 64 < n) tk_take2(best, k[c], k[c + 1], lane);     // uniform over the wave
+    for (int c = 0; c < PERW; c++) {
+        if (c * nw < (u32) MAXCH && (c * nw + wave) * 64 < n) {     // uniform over the wave; a chunk of nothing is sorted as it is
+            if (c & 1) tk_sort64<true>(k[c], lane);
+            else tk_sort64<false>(k[c], lane);
+        }
+    }
+#pragma unroll
+    for (int w = 1; w < PERW; w *= 2) {
+#pragma unroll
+        for (int c = 0; c < PERW; c += 2 * w) {
+            k[c] = tk_larger(k[c], k[c + w]);                        // ascending against descending
+            if (2 * w == PERW || ((c / (2 * w)) & 1)) tk_merge<64, true>(k[c], lane);
+            else tk_merge<64, false>(k[c], lane);
+        }
+    }
+    u64 best = k[0];
     for (u32 half = nw >> 1; half > 0; half >>= 1) {
         if (wave >= half && wave < 2 * half) sh[wave * 64 + lane] = best;
         __syncthreads();
@@ -300,8 +307,14 @@ __device__ __forceinline__ u64 tk_best_of_4096(u32 n, F key, u64* sh) {
     return best;
 }
 
+// Up to 4096 keys by 16 waves (4 chunks a wave) or 4 waves (16 chunks a wave).
+template <class F>
+__device__ __forceinline__ u64 tk_best_of_4096(u32 n, F key, u64* sh) {
+    return (blockDim.x >> 6) == 16 ? tk_best_of<64, 4>(n, key, sh) : tk_best_of<64, 16>(n, key, sh);
+}
+
 // Slice b of row r (blockIdx.x = r * nb + b): the 64 best of logits[r*stride + 4096 b .. +4096) into sv/si[(r*nb + b)*64 ..].
-// Slots past the vocabulary hold (-inf, 0xffffffff).  grid = rows * nb, block 1024 (or 256).
+// Slots past the vocabulary hold (-inf, 0xffffffff).  grid = rows * nb, block 1024 or 256.
 extern "C" __global__ void __launch_bounds__(1024) topk_slices(const float* logits, u32 vocab, u32 stride, u32 nb, float* sv, u32* si) {
     __shared__ u64 sh[1024];
     const u32 r = blockIdx.x / nb, b = blockIdx.x % nb;
@@ -318,7 +331,7 @@ extern "C" __global__ void __launch_bounds__(1024) topk_slices(const float* logi
 }
 
 // Row r = blockIdx.x: the 64 best of its nb * 64 slice winners (nb <= 64) into out[r*128 .. +64) (value bits) and
-// out[r*128 + 64 .. +64) (ids).  grid = rows, block 1024 (or 256).
+// out[r*128 + 64 .. +64) (ids).  grid = rows, block 1024 or 256.
 extern "C" __global__ void __launch_bounds__(1024) topk_merge(const float* sv, const u32* si, u32 nb, u32* out) {
     __shared__ u64 sh[1024];
     const u32 r = blockIdx.x;
@@ -501,7 +514,7 @@ extern "C" __global__ void __launch_bounds__(64) proxy_compact_seen(u32* seen, u
 // topk_slices over the packed logits of a block list (forward.cu:4626-4647): element i of row r (i < 128 sel[0]) is output
 // sel[1 + i / 128] * 128 + i % 128; elements past the list hold (-inf, 0xffffffff).  The list ascends, so packed order is
 // output order: candidates are ordered by their place and the place is turned into the output at the end.  grid = rows * nb,
-// block 1024 (or 256).
+// block 1024 or 256.
 extern "C" __global__ void __launch_bounds__(1024) topk_slices_blks(const float* logits, u32 stride, const u32* sel, u32 nb, float* sv, u32* si) {
     __shared__ u64 sh[1024];
     const u32 r = blockIdx.x / nb, b = blockIdx.x % nb;
