@@ -899,6 +899,42 @@ def test_top64_on_adversarial_rows(gpu, block):
         assert np.array_equal(words[r, :64], bits(vals)), f"row {r}"
 
 
+def test_top64_over_sizes_and_value_kinds(gpu):
+    """Vocabularies of fewer than 64 words, around a chunk, a slice and several slices; normal values, heavy ties, a mix of NaN,
+    both infinities and zeros of both signs, and a row of -inf only; both workgroup sizes: values and ids as the oracle's sort
+    gives them, unused places (-inf, 0xffffffff)."""
+    rng = np.random.default_rng(123)
+    A = sz.Arg
+    for vocab in (1, 63, 65, 4095, 4097, 12289):
+        for block in (256, 1024):
+            for kind in range(4):
+                rows = 2
+                x = rng.normal(size=(rows, vocab)).astype(np.float32)
+                if kind == 1:
+                    x = rng.integers(-3, 4, (rows, vocab)).astype(np.float32)
+                elif kind == 2:
+                    m = rng.random((rows, vocab))
+                    for lo, hi, v in ((0, 0.05, np.nan), (0.05, 0.1, -np.inf), (0.1, 0.12, np.inf), (0.12, 0.2, -0.0), (0.2, 0.28, 0.0)):
+                        x[(m >= lo) & (m < hi)] = v
+                elif kind == 3:
+                    x[:] = -np.inf
+                nb = (vocab + 4095) // 4096
+                dl = dev(gpu, x)
+                sv = gpu.empty(rows * nb * 64, dtype=gpu.float32, device="cuda")
+                si = gpu.empty(rows * nb * 64, dtype=gpu.int32, device="cuda")
+                out = gpu.empty(rows * 128, dtype=gpu.int32, device="cuda")
+                sz.launch("topk_slices", (rows * nb, 1, 1), (block, 1, 1), 0, 0,
+                          [A.ptr(dl.data_ptr()), A.u32(vocab), A.u32(vocab), A.u32(nb), A.ptr(sv.data_ptr()), A.ptr(si.data_ptr())])
+                sz.launch("topk_merge", (rows, 1, 1), (block, 1, 1), 0, 0, [A.ptr(sv.data_ptr()), A.ptr(si.data_ptr()), A.u32(nb), A.ptr(out.data_ptr())])
+                gpu.cuda.synchronize()
+                w = out.cpu().numpy().view(np.uint32).reshape(rows, 128)
+                k = min(64, vocab)
+                for r in range(rows):
+                    vals, ids = O.topk(x[r], k)
+                    assert np.array_equal(w[r, 64:64 + k], ids) and np.array_equal(w[r, :k], bits(vals)), (vocab, block, kind, r)
+                    assert np.all(w[r, 64 + k:] == 0xffffffff) and np.all(w[r, k:64] == bits(np.float32(-np.inf))), (vocab, block, kind, r)
+
+
 def test_head_top_hands_over_the_sorted_top_64(gpu):
     rng = np.random.default_rng(21)
     vocab, hidden, m = 9000, 2048, 3
