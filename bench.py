@@ -127,8 +127,9 @@ def exl3_round(torch, sz, synth, synth_device, stream, L, rates, tag):
     act_dn = pairs * 2 * FF * 2 * 4 + pairs * HIDDEN * 4           # those partials in; one down output per pair out
     w.kernel_bytes = {"head_q8_0_argmax": head_bytes + ROWS * HIDDEN * 4, "head_q8_0_argmax_mfma": head_bytes + ROWS * HIDDEN * 4}
     for kb in (2, 3, 4):
-        w.kernel_bytes["verify_gate_up_exl3_%d" % kb] = n_sel[kb] * gu_bytes[kb] + act_gu
-        w.kernel_bytes["verify_down_exl3_%d" % kb] = n_sel[kb] * dn_bytes[kb] + act_dn
+        for form in ("", "mma_", "mmaw_", "lin_", "linw_"):      # the exact launches and the matrix-core ones (sz_session_set_expert_mode)
+            w.kernel_bytes["verify_gate_up_%sexl3_%d" % (form, kb)] = n_sel[kb] * gu_bytes[kb] + act_gu
+            w.kernel_bytes["verify_down_%sexl3_%d" % (form, kb)] = n_sel[kb] * dn_bytes[kb] + act_dn
     w.step, w.check, w.set_eager = step, check, (lambda eager: sess.set_graph(not eager))
     w.step_bytes = moe_bytes + head_bytes + act_bytes
     w.counters_key = "config5" if (L == 48 and tag == "config 5" and ROWS == 4) else ("config3" if (tag == "config 3" and ROWS == 4) else None)

@@ -146,6 +146,7 @@ _SIGNATURES = {
     "sz_session_set_head": (_i32, [_vp, _i32, _u64]),
     "sz_session_set_head_proxy": (_i32, [_vp, _u32]),
     "sz_session_set_graph": (_i32, [_vp, _i32]),
+    "sz_session_set_expert_mode": (_i32, [_vp, _i32]),
     "sz_moe_layer_verify": (_i32, [_vp, _u32, _u32, _u64, _u64, _u64, _u64, _u64]),
     "sz_session_set_router": (_i32, [_vp, _u32, _i32, _u64, _i32, _u64]),
     "sz_moe_router_verify": (_i32, [_vp, _u32, _u32, _u64, _u64]),
@@ -514,6 +515,10 @@ class Session:
 
     def set_graph(self, enabled):
         check(lib().sz_session_set_graph(self._h, int(enabled)))
+
+    def set_expert_mode(self, mode):
+        """0: the exact EXL3 layer kernels, 1: the matrix cores on the codebook's f16 values, 2 (default): on the linearised codebook."""
+        check(lib().sz_session_set_expert_mode(self._h, int(mode)))
 
     def buffer(self, which):
         """Device address of a batch buffer: 0 plan, 1 gate/up partial sums, 2 down products, 3/4 GGUF rows, 5..12 the head screen's."""

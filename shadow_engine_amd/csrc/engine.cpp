@@ -332,6 +332,9 @@ struct sz_session {
     } pf;   // the prefill chunk's buffers, grown on demand
     void* top_host = nullptr;  // pinned host memory the top-64 merge writes to directly (8 rows of 128 words): no copy back
     bool last_fused = false;   // the last layer call left its routing in the fused layout [tidx | w | cnt]
+    // how an EXL3 layer at a whole bit rate multiplies (sz_session_set_expert_mode): 0 the exact kernels, a weight at a time on
+    // the vector unit; 1 the matrix cores with the codebook's own f16 values; 2 the matrix cores with the linearised codebook
+    int expert_mode = 2;
     std::map<SzGraphKey, uint64_t> graphs;
     // plan offsets for the largest batch
     uint32_t GT_max = 0;
@@ -359,6 +362,25 @@ PlanLayout plan_layout(uint32_t m, uint32_t k) {
     return p;
 }
 
+// The matrix-core EXL3 layer's plan behind [tidx | w | cnt] (verify_plan_exl3 in kernels/exl3.hip): byte offset of the item
+// list, item slots (one a pair plus the shared expert's, an even number), bytes of the whole.
+struct MmaPlan {
+    uint32_t ioff, slots, bytes;
+};
+MmaPlan mma_plan(uint32_t m, uint32_t k) {
+    MmaPlan p{};
+    p.ioff = (uint32_t) align16(2ull * m * k * 4 + m * 4);
+    p.slots = (m * k + 3) & ~1u;   // at least one more than the most items there can be: the last slot is never an item
+    p.bytes = p.ioff + 16 + p.slots * 32;
+    return p;
+}
+// Dynamic LDS of its two product launches: EXL3_MMA_LDS_WORDS there (a 4-row ring, the A rows and the scales of 4 waves).
+uint32_t mma_lds_bytes(int bits, uint32_t nmax) {
+    const uint32_t stride = (bits == 3 || bits == 4) ? 4 : (uint32_t) bits;
+    const uint32_t ring = 4 * 64 * stride;
+    return 4 * (4 * (ring + nmax * 128 + 64 + 16) + 64);
+}
+
 int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, uint64_t sgl, uint64_t y, uint64_t stream) {
     const sz_session_config& c = s->cfg;
     if (l >= s->layers.size() || !s->layers[l].set) return fail("sz_moe_layer_verify: layer " + std::to_string(l) + " has no experts set");
@@ -375,7 +397,36 @@ int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, ui
     const uint64_t addr = plan + p.a0, rec = plan + p.r0, wts = plan + p.w_off, cnt = plan + p.counts_off;
     const uint64_t addr_d = addr + 2ull * p.GT * 8, rec_d = rec + 2ull * p.GT * 17 * 4;
     const std::string kn = "matvec_grouped_" + tag;
-    if (f.exl3) {
+    if (f.exl3 && !f.half && s->expert_mode != 0) {
+        // the matrix-core layer: a plan of the batch's distinct experts, then gate/up and down with an item's tokens on the rows
+        // of the matrix instruction, then the rank-order sum (kernels/exl3.hip, "the verify layer on the matrix cores")
+        const MmaPlan mp = mma_plan(m, c.top_k);
+        const uint32_t zs_gu = (c.hidden / 128 + 3) / 4, zs_d = exl3_ksplit(c.ff);
+        const uint64_t part = matrix_bytes(f, c.hidden, c.ff);
+        if (part >> 32) return fail("sz_moe_layer_verify: a projection of 4 GiB or more");
+        const uint32_t nmax = m > 4 ? 8 : 4;
+        const uint32_t lds = mma_lds_bytes(f.bits, nmax);
+        const std::string variant = std::string(s->expert_mode == 2 ? "lin" : "mma") + (nmax == 8 ? "w" : "");
+        const std::string k1 = "verify_gate_up_" + variant + "_" + tag, k2 = "verify_down_" + variant + "_" + tag;
+        {
+            const sz_arg a[] = {P(rl), P(plan), U32(mp.ioff), U32(c.n_expert), U32(c.top_k), U32(m), U32(shared ? 1 : 0)};
+            if (launch("verify_plan_exl3", 1, 1, 1, 64 * m, 0, stream, a)) return 1;
+        }
+        {
+            const sz_arg a[] = {P(rl), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(u), P(plan), U32(mp.ioff), P(s->part.ptr),
+                                U32(c.n_expert), U32(c.top_k), U32(m), U32(c.hidden), U32(c.ff)};
+            if (launch(k1.c_str(), c.ff / 128, 2 * mp.slots, zs_gu, 256, lds, stream, a)) return 1;
+        }
+        {
+            const sz_arg a[] = {U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(plan), U32(mp.ioff), P(s->part.ptr), P(s->dn.ptr),
+                                U32(c.top_k), U32(m), U32(c.hidden), U32(c.ff), U32(zs_gu)};
+            if (launch(k2.c_str(), c.hidden / 128, mp.slots, zs_d, 256, lds, stream, a)) return 1;
+        }
+        s->last_fused = true;
+        const sz_arg a[] = {P(s->dn.ptr), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(plan), P(sgl), P(y),
+                            U32(c.top_k), U32(m), U32(c.hidden), U32(c.ff), U32(zs_d == 1 ? 0 : zs_d)};
+        return launch("verify_combine_exl3", c.hidden / 128, m, 1, zs_d == 1 ? 128 : 1024, 0, stream, a);
+    } else if (f.exl3) {
         // the fused layer: three launches, the work items are the (token, rank) pairs themselves, no plan.  A wave of
         // launch 1 takes one 128-block of the input, 4 waves a workgroup (EXL3_GU_WAVES, EXL3_VERIFY_NB in kernels/exl3.hip).
         const uint32_t S = p.G + m, zs_gu = (c.hidden / 128 + 3) / 4, zs_d = exl3_ksplit(c.ff);
@@ -620,12 +671,13 @@ sz_session* sz_session_new(const sz_session_config* cfg) {
     sz_session* s = new sz_session();
     s->cfg = c;
     s->layers.resize(c.n_layers);
+    if (const char* e = std::getenv("SHADOWZERO_EXPERT_MODE")) s->expert_mode = std::min(2, std::max(0, std::atoi(e)));
     const PlanLayout p = plan_layout(c.max_rows, c.top_k);
     s->GT_max = p.GT;
     const uint64_t ks_gu = exl3_ksplit(c.hidden), ks_d = exl3_ksplit(c.ff);
     const uint64_t part = std::max<uint64_t>(2ull * p.GT * ks_gu * 4 * c.ff, (uint64_t) p.GT * ks_d * 4 * c.hidden) * 4;
     const uint64_t nparts = c.vocab / 4 + 1;
-    bool bad = s->plan.need(p.bytes) || s->eg.need(2ull * p.R * c.ff * 4) || s->act.need((uint64_t) p.R * c.ff * 4) ||
+    bool bad = s->plan.need(std::max(p.bytes, mma_plan(c.max_rows, c.top_k).bytes)) || s->eg.need(2ull * p.R * c.ff * 4) || s->act.need((uint64_t) p.R * c.ff * 4) ||
                s->eo.need((uint64_t) p.R * c.hidden * 4) || s->part.need(part) || s->ids.need(64) ||
                s->dn.need((uint64_t) p.GT * ks_d * 4 * c.hidden * 4);
     if (c.vocab) bad = bad || s->head_part.need(nparts * 4 * 2 * 4);
@@ -784,6 +836,18 @@ uint64_t sz_session_buffer(sz_session* s, int32_t which) {
     const uint64_t at[] = {s->plan.ptr, s->part.ptr, s->dn.ptr, s->eg.ptr, s->eo.ptr, s->hp.w_q2.ptr, s->hp.w_sc.ptr, s->hp.xq.ptr, s->hp.x_sc.ptr,
                            s->hp.x_corr.ptr, s->hp.bmax.ptr, s->hp.sel.ptr, s->hp.logits.ptr};
     return which >= 0 && which < (int32_t) (sizeof at / sizeof at[0]) ? at[which] : 0;
+}
+
+int32_t sz_session_set_expert_mode(sz_session* s, int32_t mode) {
+    clear_error();
+    if (!s) return fail("sz_session_set_expert_mode: null session");
+    if (mode < 0 || mode > 2) return fail("sz_session_set_expert_mode: mode " + std::to_string(mode) + " (0 exact, 1 matrix cores, 2 matrix cores with the linearised codebook)");
+    if (s->expert_mode != mode) {
+        for (auto& g : s->graphs) sz_graph_destroy(g.second);   // a captured round holds the other mode's launches
+        s->graphs.clear();
+    }
+    s->expert_mode = mode;
+    return 0;
 }
 
 int32_t sz_session_set_graph(sz_session* s, int32_t enabled) {

@@ -1202,3 +1202,541 @@ extern "C" __global__ void __launch_bounds__(64) cols_plan(u64* wtab, u32* gtab,
         r[9 + j] = 4 * g + (j < 4 ? j : 0);
     }
 }
+
+// --------------------------------------------------------------------------------- the verify layer on the matrix cores
+// The same layer as verify_gate_up / verify_down above, for callers that accept f32 outputs within a tolerance instead of
+// the exact per-weight arithmetic (the reference's mma_grouped_exl3_K beside its exact kernels, kernels/exl3.cu:682-725,
+// held to 3e-3 of the largest output by crates/shadowzero-cuda/tests/exl3.rs:201).  Two things change.
+// (1) The work items are the DISTINCT experts of the batch, not the (token, rank) pairs: a small first launch selects every
+// token's experts and lists each expert once with the tokens that chose it, the shared expert as the first item with all of
+// them, so an expert's weights are decoded once however many tokens use it.
+// (2) The dot products run on the matrix cores, as in the head above: a lane decodes 4 consecutive weights of the bit stream,
+// a 16 x 16 tile is one B operand of v_mfma_f32_16x16x16_f16, the item's tokens ride on the A rows as f16 high and low
+// parts (8 tokens cost what one costs).  With LIN the codebook's last step is left to the end of the sum: a weight is
+// f16(h k_inv + k_bias) with h = 1024 + the byte sum, an integer that IS an f16 as the byte-sum instruction leaves it, so
+// the B operand is h itself and sum x w = k_inv sum x h + k_bias sum x, off from the exact value only by the rounding of
+// each weight to f16 that is skipped (half a unit in the last place of a weight, about 1.5e-4 of an output, relative); the
+// sum of a rotated block is sqrt(128) times the block's first element before the rotation.  Without LIN the weights are the
+// codebook's bits and only the order of the f32 additions and the 22 bits kept of an input differ from the exact kernels.
+// The plan: pbuf holds u32 tidx[m k] | f32 w[m k] | u32 cnt[m] as for the exact kernels, then at byte ioff (16-byte
+// aligned) u32 n_items, 3 unused words, and 8 words an item: expert (0xffffffff: the shared one), n tokens, their rows as
+// 8 bytes, their pair numbers as 8 u16 (pair j k + t of token j and rank t, m k + j for the shared expert: the row of the
+// partial sums and of launch 2's output, which verify_combine_exl3 reads as it does after the exact launches).
+
+// grid 1, block 64 m.  Wave j selects token j's experts (lane t < k then holds rank t's); the items come out of three tables
+// in LDS indexed by expert: the lowest pair that chose it (that pair's thread writes the item), the tokens that chose it as
+// a bit mask, and each such token's rank.  The routing weights are not needed before launch 3 and are left to a spare
+// workgroup of launch 1 (verify_route_weights below).
+extern "C" __global__ void __launch_bounds__(512) verify_plan_exl3(const float* logits, u8* pbuf, u32 ioff, u32 ne, u32 k, u32 m, u32 shared) {
+    __shared__ double ex[8 * 512];   // the exact selection's scratch, a wave's 512 doubles
+    __shared__ u32 top[8][16];
+    __shared__ u32 lowest[512];      // expert -> the lowest pair number that chose it
+    __shared__ u32 tokens[512];      // expert -> bit j: token j chose it
+    __shared__ u8 rank[512 * 8];     // expert, token -> the token's rank of it
+    __shared__ u32 wave_items[8];
+    const u32 lane = threadIdx.x & 63, j = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), G = m * k;
+    u32* tidx = (u32*) pbuf;
+    u32* plan = (u32*) (pbuf + ioff);
+    for (u32 i = threadIdx.x; i < 512; i += blockDim.x) {
+        lowest[i] = 0xffffffffu;
+        tokens[i] = 0;
+    }
+    route_ids(logits + (u64) j * ne, ne, k, lane, ex + j * 512, top[j]);
+    __syncthreads();
+    const u32 e = lane < k ? top[j][lane] : 0xffffffffu;
+    const u32 p = j * k + lane;
+    if (lane < k) tidx[p] = e;
+    if (e != 0xffffffffu) {
+        atomicMin(&lowest[e], p);
+        atomicOr(&tokens[e], 1u << j);
+        rank[e * 8 + j] = (u8) lane;
+    }
+    __syncthreads();
+    const bool isf = e != 0xffffffffu && lowest[e] == p;
+    const u64 firsts = __builtin_amdgcn_ballot_w64(isf);
+    if (lane == 0) wave_items[j] = __builtin_popcountll(firsts);
+    __syncthreads();
+    u32 slot = shared ? 1u : 0u;
+    for (u32 w = 0; w < j; w++) slot += wave_items[w];
+    if (isf) {
+        slot += __builtin_popcountll(firsts & ((1ull << lane) - 1));
+        u32 n = 0;
+        u64 toks = 0, pr0 = 0, pr1 = 0;
+        for (u32 mask = tokens[e]; mask; mask &= mask - 1) {
+            const u32 jj = __builtin_ctz(mask);
+            toks |= (u64) jj << (8 * n);
+            const u64 pv = jj * k + rank[e * 8 + jj];
+            if (n < 4) pr0 |= pv << (16 * n);
+            else pr1 |= pv << (16 * (n - 4));
+            n++;
+        }
+        u32x4* rec = (u32x4*) (plan + 4 + 8 * slot);
+        rec[0] = u32x4{e, n, (u32) toks, (u32) (toks >> 32)};
+        rec[1] = u32x4{(u32) pr0, (u32) (pr0 >> 32), (u32) pr1, (u32) (pr1 >> 32)};
+    }
+    if (threadIdx.x == 0) {
+        u32 count = shared ? 1u : 0u;
+        for (u32 w = 0; w < m; w++) count += wave_items[w];
+        plan[0] = count;
+        if (shared) {
+            u64 toks = 0, pr0 = 0, pr1 = 0;
+            for (u32 jj = 0; jj < m; jj++) {
+                toks |= (u64) jj << (8 * jj);
+                const u64 pv = G + jj;
+                if (jj < 4) pr0 |= pv << (16 * jj);
+                else pr1 |= pv << (16 * (jj - 4));
+            }
+            u32x4* rec = (u32x4*) (plan + 4);
+            rec[0] = u32x4{0xffffffffu, m, (u32) toks, (u32) (toks >> 32)};
+            rec[1] = u32x4{(u32) pr0, (u32) (pr0 >> 32), (u32) pr1, (u32) (pr1 >> 32)};
+        }
+    }
+}
+
+// The renormalised routing weights and the counts of the chosen experts tidx (pbuf, as the plan left it) into w and cnt:
+// a wave a token, for a workgroup that has nothing else to do.
+__device__ __forceinline__ void verify_route_weights(const float* __restrict__ logits, u8* __restrict__ pbuf, u32 ne, u32 k, u32 m, u32 wave, u32 lane) {
+    const u32 G = m * k;
+    for (u32 j = wave; j < m; j += 4) {
+        u32 kk;
+        const float wt = route_weights(logits + (u64) j * ne, ne, k, lane, (const u32*) pbuf + j * k, &kk);
+        if (lane < k) ((float*) (pbuf + G * 4))[j * k + lane] = wt;
+        if (lane == 0) ((u32*) (pbuf + 2 * G * 4))[j] = kk;
+    }
+}
+
+// Two states to the f16 pair (1024 + byte sum) that the codebook's multiply-add would start from.
+__device__ __forceinline__ f16x2 exl3_h_pair(u32 sa, u32 sb) {
+    const u32 lo = __builtin_amdgcn_sad_u8(exl3_mul(sa), 0u, 0x64006400u);
+    return __builtin_bit_cast(f16x2, __builtin_amdgcn_sad_hi_u8(exl3_mul(sb), 0u, lo));
+}
+
+#define EXL3_KINV 0.0067672729f    /* f16 0x1eee */
+#define EXL3_KBIAS (-10.3828125f)  /* f16 0xc931 */
+
+// A wave's A rows in LDS: f16 astrip[(tile row * 2 NMAX + A row) * 16 + slot], A row 2 r the high and 2 r + 1 the low part
+// of token r.  The lane holds elements `lane` (a0) and `lane + 64` (a1) of the token's rotated 128-block; they are scaled
+// by the power of two that takes the block's largest magnitude to [2^14, 2^15) (returned inverse undoes it).
+template <int NMAX>
+__device__ __forceinline__ float exl3_put_a_rows(u16* astrip, u32 r, float a0, float a1, u32 lane) {
+    const float mx = wave_max_f32(fmaxf(__builtin_fabsf(a0), __builtin_fabsf(a1)));
+    float scale, iv;
+    pow2_scale_of(f32_bits(mx), scale, iv);
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const u32 i = lane + 64 * h;
+        const float v = (h ? a1 : a0) * scale;
+        const _Float16 hi = (_Float16) v;
+        const _Float16 lo = (_Float16) (v - (float) hi);
+        u16* at = astrip + ((i >> 4) * (2 * NMAX) + 2 * r) * 16 + exl3_aslot(i & 15);
+        at[0] = __builtin_bit_cast(u16, hi);
+        at[16] = __builtin_bit_cast(u16, lo);
+    }
+    return iv;
+}
+
+// The decode loop of one wave on the matrix cores: the 8 tile rows of one 128-input block (requested into the ring by
+// exl3_rows_issue) against the A rows in astrip; acc[c] = the 16 x 16 sums of column tile c (row 4 a + q of the lane group
+// a = lane / 16: token 2 a high, low, token 2 a + 1 high, low; column lane % 16).
+template <int K, bool LIN, int NMAX>
+__device__ __forceinline__ void exl3_wave_mma(const u32* __restrict__ row0, u64 pitch, const u32* wb, u32 lds, const u16* astrip, u32 n, u32 lane,
+                                              f32x4 (&acc)[8]) {
+    constexpr int D = 4;
+    typedef Exl3Rows<K, D> R;
+    constexpr int stride = R::stride, ur = R::unit_rows;
+    constexpr bool one_shift = 16 + 3 * K <= 32;
+    const u32 n16 = lane & 15, a = lane >> 4;
+    const u32 t0 = 32 * (n16 & 7) + 8 * a + 4 * (n16 >> 3);
+    auto window = [&](u32 e, u32& om, u32& op, u32& sh) {
+        const u32 jp = (e - 1) >> 5, jm = (jp + 8 * K - 1) % (8 * K);
+        sh = 31 - ((e - 1) & 31);
+        om = (jm / K) * stride + jm % K;
+        op = (jp / K) * stride + jp % K;
+    };
+    u32 om1, op1, sh1, om0 = 0, op0 = 0, sh0 = 0;
+    window((t0 + 4) * K, om1, op1, sh1);
+    if constexpr (!one_shift) window((t0 + 2) * K, om0, op0, sh0);
+#pragma unroll
+    for (int c = 0; c < 8; c++) acc[c] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    const bool fed = n16 < 2 * n;                          // this lane supplies A row n16
+    const u16* xa0 = astrip + (fed ? n16 : 0) * 16 + 4 * a;
+#pragma unroll 1
+    for (u32 i = 0; i < 8; i++) {
+        exl3_rows_wait<K, D>(i + D > 8 ? i + D - 8 : 0);
+        const u32* row = wb + (i & (D - 1)) * R::row_words;
+        u32 w1[8][2], w0[8][2];
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            w1[c][0] = row[c * 8 * stride + om1];
+            w1[c][1] = row[c * 8 * stride + op1];
+            if constexpr (!one_shift) {
+                w0[c][0] = row[c * 8 * stride + om0];
+                w0[c][1] = row[c * 8 * stride + op0];
+            }
+        }
+        typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+        u32x2 xv = *(const u32x2*) (xa0 + i * (2 * NMAX * 16));
+        if (!fed) xv = u32x2{0u, 0u};
+        if ((i + 1) % ur == 0 && i + D + 1 - ur < 8) {
+            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): the row's words are in registers, its slot can take the row D further on
+            exl3_unit_issue<K, D>(row0, pitch, i + D + 1 - ur, lane, lds);
+        }
+        const f16x4 av = __builtin_bit_cast(f16x4, xv);
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            const u32 hi = __builtin_amdgcn_alignbit(w1[c][0], w1[c][1], sh1);
+            u32 s0, s1;
+            if constexpr (one_shift) {
+                s0 = __builtin_amdgcn_ubfe(hi, 3 * K, 16);
+                s1 = __builtin_amdgcn_ubfe(hi, 2 * K, 16);
+            } else {
+                const u32 lo = __builtin_amdgcn_alignbit(w0[c][0], w0[c][1], sh0);
+                s0 = __builtin_amdgcn_ubfe(lo, K, 16);
+                s1 = lo & 0xffffu;
+            }
+            const u32 s2 = __builtin_amdgcn_ubfe(hi, K, 16), s3 = hi & 0xffffu;
+            const f16x2 b01 = LIN ? exl3_h_pair(s0, s1) : exl3_cb2_pair(s0, s1), b23 = LIN ? exl3_h_pair(s2, s3) : exl3_cb2_pair(s2, s3);
+            const f16x4 bv = {b01[0], b01[1], b23[0], b23[1]};
+            acc[c] = __builtin_amdgcn_mfma_f32_16x16x16f16(av, bv, acc[c], 0, 0, 0);
+        }
+    }
+}
+
+// What a wave leaves for the workgroup's sum: red[(wave * NMAX + r) * 128 + column] = token r's partial sum of the wave's
+// 128 inputs (high + low part, scale undone; with LIN times k_inv plus the token's k_bias term).  iv[h], cr[h]: the inverse
+// scale and the k_bias term of the lane group's tokens 2 a + h.
+template <bool LIN, int NMAX>
+__device__ __forceinline__ void exl3_mma_to_red(float* red, u32 wave, u32 n, u32 lane, const f32x4 (&acc)[8], const float (&iv)[2], const float (&cr)[2]) {
+    const u32 n16 = lane & 15, a = lane >> 4;
+#pragma unroll
+    for (int h = 0; h < 2; h++) {
+        const u32 r = 2 * a + h;
+        if (r < n && r < (u32) NMAX) {
+            const float f = iv[h] * (LIN ? EXL3_KINV : 1.0f), c0 = LIN ? cr[h] : 0.0f;
+            float* o = red + (wave * NMAX + r) * 128 + n16;
+#pragma unroll
+            for (int c = 0; c < 8; c++) o[16 * c] = __builtin_fmaf(acc[c][2 * h] + acc[c][2 * h + 1], f, c0);
+        }
+    }
+}
+
+// The LDS a workgroup of the two launches needs, in words, for ring rows of `ring` words a wave (Exl3Rows<K, 4>::words).
+#define EXL3_MMA_WAVE_WORDS(ring, NMAX) ((ring) + (NMAX) * 128 + 64 + 16)   /* ring, A rows, input scales, the tokens' inverse scales and k_bias terms */
+#define EXL3_MMA_LDS_WORDS(ring, NMAX) (4 * EXL3_MMA_WAVE_WORDS(ring, NMAX) + 64)
+
+// Launch 1: the gate and up products of every item, partial sums gup[((sel * S + pair) * zs + z)][ff] as the exact launch
+// leaves them (already through the output-side transform and scales).  grid = (ff / 128, 2 IT, zs), IT = the item slots
+// (an even number above m k + 1), zs = ceil(hidden / 512); block 256; dynamic LDS EXL3_MMA_LDS_WORDS.
+template <int K, bool LIN, int NMAX>
+__device__ __forceinline__ void verify_gate_up_mma_kernel(const float* __restrict__ logits, u64 ebase, u64 estride, u64 shbase, u32 part,
+                                                          const float* __restrict__ u, u8* __restrict__ pbuf, u32 ioff, float* __restrict__ gup, u32 ne,
+                                                          u32 k, u32 m, u32 hidden, u32 ff) {
+    constexpr int D = 4;
+    typedef Exl3Rows<K, D> R;
+    constexpr int WW = EXL3_MMA_WAVE_WORDS(R::words, NMAX);
+    extern __shared__ __attribute__((aligned(16))) u32 dyn[];
+    const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const u32 IT = gridDim.y >> 1, sel = blockIdx.y >= IT ? 1u : 0u, it = blockIdx.y - sel * IT;
+    const u32* plan = (const u32*) (pbuf + ioff);
+    if (it >= plan[0]) {
+        // the last item slot is never an item (there are at most m k + 1): one of its workgroups works the routing weights out
+        // for launch 3 while the others multiply
+        if (blockIdx.y == gridDim.y - 1 && blockIdx.x == 0 && blockIdx.z == 0) verify_route_weights(logits, pbuf, ne, k, m, wave, lane);
+        return;
+    }
+    const u32* rec = plan + 4 + 8 * it;
+    const u32 e = rec[0], n = min(rec[1], (u32) NMAX);
+    const u64 toks = (u64) rec[2] | ((u64) rec[3] << 32);
+    const u32 S = m * k + m;
+    const u8* bp = (const u8*) (e == 0xffffffffu ? shbase : ebase + e * estride) + (u64) sel * part;
+    const u32 kbs = hidden / 128, kb = blockIdx.z * 4 + wave;
+    const bool live = kb < kbs;
+    u32* wring = dyn + wave * WW;
+    u16* astrip = (u16*) (wring + R::words);
+    u32* sc = wring + R::words + NMAX * 128;
+    u32* sv_out = dyn + 4 * WW;
+    float iv[2] = {0.0f, 0.0f}, cr[2] = {0.0f, 0.0f};   // the inverse scales and the k_bias terms of the lane group's two tokens
+    f32x4 acc[8];
+    if (live) {
+        float v[NMAX][2];
+#pragma unroll
+        for (int r = 0; r < NMAX; r++) {
+            const u32 tok = (u32) (toks >> (8 * min((u32) r, n - 1))) & 0xffu;
+            const float* xj = u + (u64) tok * hidden + kb * 128;
+            v[r][0] = xj[lane];
+            v[r][1] = xj[lane + 64];
+        }
+#pragma unroll
+        for (int r = 0; r < NMAX; r++) asm volatile("" : "+v"(v[r][0]), "+v"(v[r][1]));   // no ordinary load is in flight from now on
+        const u32 sc_lds = __builtin_amdgcn_readfirstlane(lds_offset(sc));
+        const u32 wb_lds = __builtin_amdgcn_readfirstlane(lds_offset(wring));
+        lds_load<4>(bp + kb * 256 + lane * 4, sc_lds);
+        if (wave == 0) lds_load<4>(bp + 2 * (u64) hidden + blockIdx.x * 256 + lane * 4, __builtin_amdgcn_readfirstlane(lds_offset(sv_out)));
+        const u32* row0 = (const u32*) (bp + 2 * (u64) hidden + 2 * (u64) ff + 4) + ((u64) kb * 8 * (ff / 16) + blockIdx.x * 8) * EXL3_TILE_WORDS(K, false);
+        const u64 pitch = (u64) (ff / 16) * EXL3_TILE_WORDS(K, false);
+        exl3_rows_issue<K, D>(row0, pitch, lane, wb_lds);
+        wait_vm<R::loads>();
+        const u16* sch = (const u16*) sc;
+        const float s0 = f16_to_f32(sch[lane]), s1 = f16_to_f32(sch[lane + 64]);
+        // a token's inverse scale and k_bias term wait in LDS for the lanes that hold the token's sums at the end
+        float* ivs = (float*) (sc + 64);
+#pragma unroll
+        for (int r = 0; r < NMAX; r++) {
+            if ((u32) r < n) {
+                float a0 = v[r][0] * s0, a1 = v[r][1] * s1;
+                const float c0 = (EXL3_KBIAS * 11.3137085f) * bits_f32(__builtin_amdgcn_readlane(f32_bits(a0), 0));
+                wht128_wave(a0, a1, lane);
+                const float i0 = exl3_put_a_rows<NMAX>(astrip, r, a0, a1, lane);
+                if (lane == 0) {
+                    ivs[r] = i0;
+                    ivs[NMAX + r] = c0;
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        exl3_wave_mma<K, LIN, NMAX>(row0, pitch, wring, wb_lds, astrip, n, lane, acc);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const u32 r = min(2 * (lane >> 4) + h, (u32) NMAX - 1);
+            iv[h] = ivs[r];
+            cr[h] = ivs[NMAX + r];
+        }
+    }
+    __syncthreads();   // every wave is done with its ring and A rows: the space takes the sums
+    float* red = (float*) dyn;
+    if (live) exl3_mma_to_red<LIN, NMAX>(red, wave, n, lane, acc, iv, cr);
+    __syncthreads();
+    const u32 nw = min(4u, kbs - blockIdx.z * 4);
+    const u16* sv = (const u16*) sv_out;
+    for (u32 r = wave; r < n; r += 4) {
+        float a0 = 0.0f, a1 = 0.0f;
+        for (u32 w = 0; w < nw; w++) {
+            a0 += red[(w * NMAX + r) * 128 + lane];
+            a1 += red[(w * NMAX + r) * 128 + lane + 64];
+        }
+        wht128_wave(a0, a1, lane);
+        const u32 pair = (rec[4 + (r >> 1)] >> (16 * (r & 1))) & 0xffffu;
+        float* o = gup + (((u64) sel * S + pair) * gridDim.z + blockIdx.z) * ff + blockIdx.x * 128;
+        __builtin_nontemporal_store(a0 * f16_to_f32(sv[lane]), &o[lane]);
+        __builtin_nontemporal_store(a1 * f16_to_f32(sv[lane + 64]), &o[lane + 64]);
+    }
+}
+
+// Launch 2: act = silu(gate) * up of every token of the item from launch 1's partial sums (by every wave for its own
+// 128-block, as the exact launch does), then the down product: finished blocks dn[pair][hidden] when one workgroup holds
+// the whole sum over the inputs (ff <= 512), else partial sums dn[pair * gridDim.z + z][hidden] for verify_combine_exl3.
+// grid = (hidden / 128, IT, ceil(ff / 512)), block 256, dynamic LDS as launch 1.
+template <int K, bool LIN, int NMAX>
+__device__ __forceinline__ void verify_down_mma_kernel(u64 ebase, u64 estride, u64 shbase, u32 part, const u8* __restrict__ pbuf, u32 ioff,
+                                                       const float* __restrict__ gup, float* __restrict__ dn, u32 k, u32 m, u32 hidden, u32 ff, u32 zs) {
+    constexpr int D = 4;
+    typedef Exl3Rows<K, D> R;
+    constexpr int WW = EXL3_MMA_WAVE_WORDS(R::words, NMAX);
+    extern __shared__ __attribute__((aligned(16))) u32 dyn[];
+    const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const u32 it = blockIdx.y;
+    const u32* plan = (const u32*) (pbuf + ioff);
+    if (it >= plan[0]) return;
+    const u32* rec = plan + 4 + 8 * it;
+    const u32 e = rec[0], n = min(rec[1], (u32) NMAX);
+    const u32 S = m * k + m;
+    const u8* down = (const u8*) (e == 0xffffffffu ? shbase : ebase + e * estride) + 2 * (u64) part;
+    const u32 kbs = ff / 128, kb = blockIdx.z * 4 + wave;
+    const bool live = kb < kbs;
+    u32* wring = dyn + wave * WW;
+    u16* astrip = (u16*) (wring + R::words);
+    u32* sc = wring + R::words + NMAX * 128;
+    u32* sv_out = dyn + 4 * WW;
+    float iv[2] = {0.0f, 0.0f}, cr[2] = {0.0f, 0.0f};   // the inverse scales and the k_bias terms of the lane group's two tokens
+    f32x4 acc[8];
+    if (live) {
+        // the sums of launch 1's partials of the wave's block of gate and up, every token's loads on their way at once (in
+        // two lots of four tokens when there may be more)
+        float gu[NMAX][4];
+#pragma unroll
+        for (int r0 = 0; r0 < NMAX; r0 += 4) {
+            if (r0 > 0 && n <= (u32) r0) break;
+            float pv[4][4][4];
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const u32 r = min((u32) (r0 + q), n - 1);
+                const u32 pair = (rec[4 + (r >> 1)] >> (16 * (r & 1))) & 0xffffu;
+#pragma unroll
+                for (int z = 0; z < 4; z++) {
+                    const u32 zz = min((u32) z, zs - 1);
+                    const float* pg = gup + ((u64) pair * zs + zz) * ff + kb * 128;
+                    const float* pu = gup + ((u64) (S + pair) * zs + zz) * ff + kb * 128;
+                    pv[q][z][0] = pg[lane];
+                    pv[q][z][1] = pg[lane + 64];
+                    pv[q][z][2] = pu[lane];
+                    pv[q][z][3] = pu[lane + 64];
+                }
+            }
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+#pragma unroll
+                for (int c = 0; c < 4; c++) {
+                    float t = pv[q][0][c];
+#pragma unroll
+                    for (int z = 1; z < 4; z++)
+                        if ((u32) z < zs) t += pv[q][z][c];
+                    gu[r0 + q][c] = t;
+                }
+                if (zs > 4) {
+                    const u32 r = min((u32) (r0 + q), n - 1);
+                    const u32 pair = (rec[4 + (r >> 1)] >> (16 * (r & 1))) & 0xffffu;
+                    for (u32 z = 4; z < zs; z++) {
+                        const float* pg = gup + ((u64) pair * zs + z) * ff + kb * 128;
+                        const float* pu = gup + ((u64) (S + pair) * zs + z) * ff + kb * 128;
+                        gu[r0 + q][0] += pg[lane];
+                        gu[r0 + q][1] += pg[lane + 64];
+                        gu[r0 + q][2] += pu[lane];
+                        gu[r0 + q][3] += pu[lane + 64];
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int r = 0; r < NMAX; r++) asm volatile("" : "+v"(gu[r][0]), "+v"(gu[r][1]), "+v"(gu[r][2]), "+v"(gu[r][3]));   // no ordinary load is in flight from now on
+        const u32 sc_lds = __builtin_amdgcn_readfirstlane(lds_offset(sc));
+        const u32 wb_lds = __builtin_amdgcn_readfirstlane(lds_offset(wring));
+        lds_load<4>(down + kb * 256 + lane * 4, sc_lds);
+        if (wave == 0) lds_load<4>(down + 2 * (u64) ff + blockIdx.x * 256 + lane * 4, __builtin_amdgcn_readfirstlane(lds_offset(sv_out)));
+        const u32* row0 = (const u32*) (down + 2 * (u64) ff + 2 * (u64) hidden + 4) + ((u64) kb * 8 * (hidden / 16) + blockIdx.x * 8) * EXL3_TILE_WORDS(K, false);
+        const u64 pitch = (u64) (hidden / 16) * EXL3_TILE_WORDS(K, false);
+        exl3_rows_issue<K, D>(row0, pitch, lane, wb_lds);
+        wait_vm<R::loads>();
+        const u16* sch = (const u16*) sc;
+        const float s0 = f16_to_f32(sch[lane]), s1 = f16_to_f32(sch[lane + 64]);
+        // a token's inverse scale and k_bias term wait in LDS for the lanes that hold the token's sums at the end
+        float* ivs = (float*) (sc + 64);
+#pragma unroll
+        for (int r = 0; r < NMAX; r++) {
+            if ((u32) r < n) {
+                float a0 = (siluf_ref(gu[r][0]) * gu[r][2]) * s0, a1 = (siluf_ref(gu[r][1]) * gu[r][3]) * s1;
+                const float c0 = (EXL3_KBIAS * 11.3137085f) * bits_f32(__builtin_amdgcn_readlane(f32_bits(a0), 0));
+                wht128_wave(a0, a1, lane);
+                const float i0 = exl3_put_a_rows<NMAX>(astrip, r, a0, a1, lane);
+                if (lane == 0) {
+                    ivs[r] = i0;
+                    ivs[NMAX + r] = c0;
+                }
+            }
+        }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        exl3_wave_mma<K, LIN, NMAX>(row0, pitch, wring, wb_lds, astrip, n, lane, acc);
+#pragma unroll
+        for (int h = 0; h < 2; h++) {
+            const u32 r = min(2 * (lane >> 4) + h, (u32) NMAX - 1);
+            iv[h] = ivs[r];
+            cr[h] = ivs[NMAX + r];
+        }
+    }
+    __syncthreads();
+    float* red = (float*) dyn;
+    if (live) exl3_mma_to_red<LIN, NMAX>(red, wave, n, lane, acc, iv, cr);
+    __syncthreads();
+    const u32 nw = min(4u, kbs - blockIdx.z * 4);
+    const u16* sv = (const u16*) sv_out;
+    for (u32 r = wave; r < n; r += 4) {
+        float a0 = 0.0f, a1 = 0.0f;
+        for (u32 w = 0; w < nw; w++) {
+            a0 += red[(w * NMAX + r) * 128 + lane];
+            a1 += red[(w * NMAX + r) * 128 + lane + 64];
+        }
+        const u32 pair = (rec[4 + (r >> 1)] >> (16 * (r & 1))) & 0xffffu;
+        if (gridDim.z == 1) {
+            wht128_wave(a0, a1, lane);
+            float* o = dn + (u64) pair * hidden + blockIdx.x * 128;
+            __builtin_nontemporal_store(a0 * f16_to_f32(sv[lane]), &o[lane]);
+            __builtin_nontemporal_store(a1 * f16_to_f32(sv[lane + 64]), &o[lane + 64]);
+        } else {
+            float* o = dn + ((u64) pair * gridDim.z + blockIdx.z) * hidden + blockIdx.x * 128;
+            o[lane] = a0;
+            o[lane + 64] = a1;
+        }
+    }
+}
+
+// Entry points: _mma_ the codebook's own f16 values, _lin_ the linearised form; the w variants take up to 8 tokens an item
+// (batches of more than 4 rows), the others 4.  5 workgroups of 4 waves a CU: the register budget follows it.
+#define EXL3_MMA_ENTRIES(K)                                                                                                            \
+    extern "C" __global__ void __launch_bounds__(256, 5) verify_gate_up_mma_exl3_##K(const float* logits, u64 ebase, u64 estride, u64 shbase, u32 part, const float* u, \
+                                                                                          u8* pbuf, u32 ioff, float* gup, u32 ne, u32 k, u32 m, u32 hidden, \
+                                                                                          u32 ff) {                                      \
+        verify_gate_up_mma_kernel<K, false, 4>(logits, ebase, estride, shbase, part, u, pbuf, ioff, gup, ne, k, m, hidden, ff);                     \
+    }                                                                                                                                    \
+    extern "C" __global__ void __launch_bounds__(256, 5) verify_down_mma_exl3_##K(u64 ebase, u64 estride, u64 shbase, u32 part, const u8* pbuf, \
+                                                                                       u32 ioff, const float* gup, float* dn, u32 k, u32 m, u32 hidden, \
+                                                                                       u32 ff, u32 zs) {                                 \
+        verify_down_mma_kernel<K, false, 4>(ebase, estride, shbase, part, pbuf, ioff, gup, dn, k, m, hidden, ff, zs);                   \
+    }
+#define EXL3_MMAW_ENTRIES(K)                                                                                                            \
+    extern "C" __global__ void __launch_bounds__(256, 5) verify_gate_up_mmaw_exl3_##K(const float* logits, u64 ebase, u64 estride, u64 shbase, u32 part, const float* u, \
+                                                                                          u8* pbuf, u32 ioff, float* gup, u32 ne, u32 k, u32 m, u32 hidden, \
+                                                                                          u32 ff) {                                      \
+        verify_gate_up_mma_kernel<K, false, 8>(logits, ebase, estride, shbase, part, u, pbuf, ioff, gup, ne, k, m, hidden, ff);                     \
+    }                                                                                                                                    \
+    extern "C" __global__ void __launch_bounds__(256, 5) verify_down_mmaw_exl3_##K(u64 ebase, u64 estride, u64 shbase, u32 part, const u8* pbuf, \
+                                                                                       u32 ioff, const float* gup, float* dn, u32 k, u32 m, u32 hidden, \
+                                                                                       u32 ff, u32 zs) {                                 \
+        verify_down_mma_kernel<K, false, 8>(ebase, estride, shbase, part, pbuf, ioff, gup, dn, k, m, hidden, ff, zs);                   \
+    }
+#define EXL3_LIN_ENTRIES(K)                                                                                                            \
+    extern "C" __global__ void __launch_bounds__(256, 5) verify_gate_up_lin_exl3_##K(const float* logits, u64 ebase, u64 estride, u64 shbase, u32 part, const float* u, \
+                                                                                          u8* pbuf, u32 ioff, float* gup, u32 ne, u32 k, u32 m, u32 hidden, \
+                                                                                          u32 ff) {                                      \
+        verify_gate_up_mma_kernel<K, true, 4>(logits, ebase, estride, shbase, part, u, pbuf, ioff, gup, ne, k, m, hidden, ff);                     \
+    }                                                                                                                                    \
+    extern "C" __global__ void __launch_bounds__(256, 5) verify_down_lin_exl3_##K(u64 ebase, u64 estride, u64 shbase, u32 part, const u8* pbuf, \
+                                                                                       u32 ioff, const float* gup, float* dn, u32 k, u32 m, u32 hidden, \
+                                                                                       u32 ff, u32 zs) {                                 \
+        verify_down_mma_kernel<K, true, 4>(ebase, estride, shbase, part, pbuf, ioff, gup, dn, k, m, hidden, ff, zs);                   \
+    }
+#define EXL3_LINW_ENTRIES(K)                                                                                                            \
+    extern "C" __global__ void __launch_bounds__(256, 5) verify_gate_up_linw_exl3_##K(const float* logits, u64 ebase, u64 estride, u64 shbase, u32 part, const float* u, \
+                                                                                          u8* pbuf, u32 ioff, float* gup, u32 ne, u32 k, u32 m, u32 hidden, \
+                                                                                          u32 ff) {                                      \
+        verify_gate_up_mma_kernel<K, true, 8>(logits, ebase, estride, shbase, part, u, pbuf, ioff, gup, ne, k, m, hidden, ff);                     \
+    }                                                                                                                                    \
+    extern "C" __global__ void __launch_bounds__(256, 5) verify_down_linw_exl3_##K(u64 ebase, u64 estride, u64 shbase, u32 part, const u8* pbuf, \
+                                                                                       u32 ioff, const float* gup, float* dn, u32 k, u32 m, u32 hidden, \
+                                                                                       u32 ff, u32 zs) {                                 \
+        verify_down_mma_kernel<K, true, 8>(ebase, estride, shbase, part, pbuf, ioff, gup, dn, k, m, hidden, ff, zs);                   \
+    }
+EXL3_MMA_ENTRIES(1)
+EXL3_MMA_ENTRIES(2)
+EXL3_MMA_ENTRIES(3)
+EXL3_MMA_ENTRIES(4)
+EXL3_MMA_ENTRIES(5)
+EXL3_MMA_ENTRIES(6)
+EXL3_MMA_ENTRIES(7)
+EXL3_MMA_ENTRIES(8)
+EXL3_MMAW_ENTRIES(1)
+EXL3_MMAW_ENTRIES(2)
+EXL3_MMAW_ENTRIES(3)
+EXL3_MMAW_ENTRIES(4)
+EXL3_MMAW_ENTRIES(5)
+EXL3_MMAW_ENTRIES(6)
+EXL3_MMAW_ENTRIES(7)
+EXL3_MMAW_ENTRIES(8)
+EXL3_LIN_ENTRIES(1)
+EXL3_LIN_ENTRIES(2)
+EXL3_LIN_ENTRIES(3)
+EXL3_LIN_ENTRIES(4)
+EXL3_LIN_ENTRIES(5)
+EXL3_LIN_ENTRIES(6)
+EXL3_LIN_ENTRIES(7)
+EXL3_LIN_ENTRIES(8)
+EXL3_LINW_ENTRIES(1)
+EXL3_LINW_ENTRIES(2)
+EXL3_LINW_ENTRIES(3)
+EXL3_LINW_ENTRIES(4)
+EXL3_LINW_ENTRIES(5)
+EXL3_LINW_ENTRIES(6)
+EXL3_LINW_ENTRIES(7)
+EXL3_LINW_ENTRIES(8)
