@@ -168,11 +168,13 @@ int32_t sz_session_set_head(sz_session*, int32_t ggml_type, uint64_t w);
 int32_t sz_session_set_head_proxy(sz_session*, uint32_t k_blk);
 /* How a layer of EXL3 experts at a whole bit rate multiplies in sz_moe_layer_verify, sz_moe_block_verify and sz_verify_round
  * (the reference's choice between its exact kernels and mma_grouped_exl3_K, kernels/exl3.cu:682-725, which `--exact` and
- * `tensor_prompt` make, session.rs:1741, 1817): 0 the exact kernels (every weight the codebook's f16, f32 multiply-adds in
- * input order); 1 the matrix cores on the codebook's own f16 values (only the order of the f32 additions differs); 2, the
- * default, the matrix cores on the linearised codebook (a weight's rounding to f16 is skipped: outputs within 1e-3 relative
- * L2 of the exact ones, about 2e-4 measured).  Routing ids, their order and the weights are the same bits in every mode.
- * Half-integer rates always take the exact kernels.  Environment SHADOWZERO_EXPERT_MODE sets a new session's mode. */
+ * `tensor_prompt` make, session.rs:1741, 1817): 0, the default, the exact kernels (every weight the codebook's f16, f32
+ * multiply-adds in input order, a work item a (token, expert) pair); 1 the matrix cores on the codebook's own f16 values, a
+ * work item a distinct expert with its tokens on the rows of the matrix instruction (only the order of the f32 additions and
+ * the 22 bits kept of an input differ); 2 the matrix cores on the linearised codebook (a weight's rounding to f16 is skipped:
+ * outputs within 1e-3 relative L2 of the exact ones, about 4e-4 measured).  Routing ids, their order and the weights are the
+ * same bits in every mode.  Half-integer rates always take the exact kernels.  On an MI355X the exact kernels are the fastest
+ * for batches of up to 8 rows.  Environment SHADOWZERO_EXPERT_MODE sets a new session's mode. */
 int32_t sz_session_set_expert_mode(sz_session*, int32_t mode);
 /* 0: sz_verify_round launches its kernels one by one instead of replaying a captured graph (default 1). */
 int32_t sz_session_set_graph(sz_session*, int32_t enabled);

@@ -285,8 +285,8 @@ def kernels():
     out = []
     for i in range(L.sz_kernel_count()):
         name, file, n = C.c_char_p(), C.c_char_p(), _i32()
-        kinds = (_i32 * 16)()
-        check(L.sz_kernel_info(i, C.byref(name), C.byref(file), C.byref(n), kinds, 16))
+        kinds = (_i32 * 24)()
+        check(L.sz_kernel_info(i, C.byref(name), C.byref(file), C.byref(n), kinds, 24))
         out.append((name.value.decode(), file.value.decode(), list(kinds[:n.value])))
     return out
 
@@ -517,7 +517,7 @@ class Session:
         check(lib().sz_session_set_graph(self._h, int(enabled)))
 
     def set_expert_mode(self, mode):
-        """0: the exact EXL3 layer kernels, 1: the matrix cores on the codebook's f16 values, 2 (default): on the linearised codebook."""
+        """0 (default): the exact EXL3 layer kernels, 1: the matrix cores on the codebook's f16 values, 2: on the linearised codebook."""
         check(lib().sz_session_set_expert_mode(self._h, int(mode)))
 
     def buffer(self, which):

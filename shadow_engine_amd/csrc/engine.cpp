@@ -334,7 +334,9 @@ struct sz_session {
     bool last_fused = false;   // the last layer call left its routing in the fused layout [tidx | w | cnt]
     // how an EXL3 layer at a whole bit rate multiplies (sz_session_set_expert_mode): 0 the exact kernels, a weight at a time on
     // the vector unit; 1 the matrix cores with the codebook's own f16 values; 2 the matrix cores with the linearised codebook
-    int expert_mode = 2;
+    int expert_mode = 0;
+    DevBuf plan2;              // a round's layers alternate between two plans: the sum of a layer rides the next layer's first launch, which writes that layer's routing
+    uint64_t last_plan = 0;    // the plan the last layer call left its routing in
     std::map<SzGraphKey, uint64_t> graphs;
     // plan offsets for the largest batch
     uint32_t GT_max = 0;
@@ -381,7 +383,24 @@ uint32_t mma_lds_bytes(int bits, uint32_t nmax) {
     return 4 * (4 * (ring + nmax * 128 + 64 + 16) + 64);
 }
 
-int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, uint64_t sgl, uint64_t y, uint64_t stream) {
+// The rank-order sum of an EXL3 layer that has not been launched yet: inside sz_verify_round it rides the first launch of
+// the layer after it (whose routing goes to the session's other plan buffer), and the last layer's gets a launch of its own.
+struct PendingSum {
+    bool active = false;
+    uint64_t plan = 0, sgl = 0, y = 0;
+    bool shared = false;
+};
+
+int launch_pending_sum(sz_session* s, PendingSum& ps, uint32_t m, uint64_t stream) {
+    if (!ps.active) return 0;
+    const sz_session_config& c = s->cfg;
+    ps.active = false;
+    const sz_arg a[] = {P(s->dn.ptr), U64(0), U64(0), U64(ps.shared ? 1 : 0), U32(0), P(ps.plan), P(ps.sgl), P(ps.y),
+                        U32(c.top_k), U32(m), U32(c.hidden), U32(c.ff), U32(0)};
+    return launch("verify_combine_exl3", c.hidden / 128, m, 1, 128, 0, stream, a);
+}
+
+int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, uint64_t sgl, uint64_t y, uint64_t stream, PendingSum* ride = nullptr) {
     const sz_session_config& c = s->cfg;
     if (l >= s->layers.size() || !s->layers[l].set) return fail("sz_moe_layer_verify: layer " + std::to_string(l) + " has no experts set");
     if (m == 0 || m > c.max_rows) return fail("sz_moe_layer_verify: " + std::to_string(m) + " rows (1.." + std::to_string(c.max_rows) + ")");
@@ -393,10 +412,30 @@ int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, ui
     const bool shared = L.shared != 0;
     if (shared && L.shared_type != L.type) return fail("the shared expert must have the routed experts' type (layer " + std::to_string(l) + ")");
     const PlanLayout p = plan_layout(m, c.top_k);
-    const uint64_t plan = s->plan.ptr;
+    // a layer whose sum may ride the next launch takes the plan buffer the pending sum is not reading
+    const uint64_t plan = (ride && ride->active && ride->plan == s->plan.ptr) ? s->plan2.ptr : s->plan.ptr;
+    s->last_plan = plan;
     const uint64_t addr = plan + p.a0, rec = plan + p.r0, wts = plan + p.w_off, cnt = plan + p.counts_off;
     const uint64_t addr_d = addr + 2ull * p.GT * 8, rec_d = rec + 2ull * p.GT * 17 * 4;
     const std::string kn = "matvec_grouped_" + tag;
+    if (ride && ride->active && !f.exl3 && launch_pending_sum(s, *ride, m, stream)) return 1;   // only an EXL3 layer's first launch carries a sum
+    // the sum of the layer before, if it rides this layer's first launch: the workgroups it adds, its arguments
+    const bool carry = f.exl3 && ride && ride->active;
+    const uint32_t carry_groups = carry ? c.hidden / 128 * m : 0;
+    const uint64_t c_plan = carry ? ride->plan : 0, c_sgl = carry ? ride->sgl : 0, c_y = carry ? ride->y : 0;
+    const uint32_t c_mode = carry ? (ride->shared ? 2 : 1) : 0;
+    // this layer's own sum: left for the next launch to carry when the caller takes care of it (launch 2 must have finished the blocks)
+    auto sum = [&](uint32_t zs_d, uint64_t part) -> int {
+        if (ride) ride->active = false;
+        s->last_fused = true;
+        if (ride && zs_d == 1) {
+            *ride = PendingSum{true, plan, sgl, y, shared};
+            return 0;
+        }
+        const sz_arg a[] = {P(s->dn.ptr), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(plan), P(sgl), P(y),
+                            U32(c.top_k), U32(m), U32(c.hidden), U32(c.ff), U32(zs_d == 1 ? 0 : zs_d)};
+        return launch("verify_combine_exl3", c.hidden / 128, m, 1, zs_d == 1 ? 128 : 1024, 0, stream, a);   // zs_d == 1: launch 2 finished the blocks
+    };
     if (f.exl3 && !f.half && s->expert_mode != 0) {
         // the matrix-core layer: a plan of the batch's distinct experts, then gate/up and down with an item's tokens on the rows
         // of the matrix instruction, then the rank-order sum (kernels/exl3.hip, "the verify layer on the matrix cores")
@@ -409,8 +448,9 @@ int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, ui
         const std::string variant = std::string(s->expert_mode == 2 ? "lin" : "mma") + (nmax == 8 ? "w" : "");
         const std::string k1 = "verify_gate_up_" + variant + "_" + tag, k2 = "verify_down_" + variant + "_" + tag;
         {
-            const sz_arg a[] = {P(rl), P(plan), U32(mp.ioff), U32(c.n_expert), U32(c.top_k), U32(m), U32(shared ? 1 : 0)};
-            if (launch("verify_plan_exl3", 1, 1, 1, 64 * m, 0, stream, a)) return 1;
+            const sz_arg a[] = {P(rl), P(plan), U32(mp.ioff), U32(c.n_expert), U32(c.top_k), U32(m), U32(shared ? 1 : 0), U32(c.hidden),
+                                P(s->dn.ptr), P(c_plan), P(c_sgl), P(c_y), U32(c_mode)};
+            if (launch("verify_plan_exl3", 1 + carry_groups, 1, 1, 64 * m, 0, stream, a)) return 1;
         }
         {
             const sz_arg a[] = {P(rl), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(u), P(plan), U32(mp.ioff), P(s->part.ptr),
@@ -422,10 +462,7 @@ int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, ui
                                 U32(c.top_k), U32(m), U32(c.hidden), U32(c.ff), U32(zs_gu)};
             if (launch(k2.c_str(), c.hidden / 128, mp.slots, zs_d, 256, lds, stream, a)) return 1;
         }
-        s->last_fused = true;
-        const sz_arg a[] = {P(s->dn.ptr), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(plan), P(sgl), P(y),
-                            U32(c.top_k), U32(m), U32(c.hidden), U32(c.ff), U32(zs_d == 1 ? 0 : zs_d)};
-        return launch("verify_combine_exl3", c.hidden / 128, m, 1, zs_d == 1 ? 128 : 1024, 0, stream, a);
+        return sum(zs_d, part);
     } else if (f.exl3) {
         // the fused layer: three launches, the work items are the (token, rank) pairs themselves, no plan.  A wave of
         // launch 1 takes one 128-block of the input, 4 waves a workgroup (EXL3_GU_WAVES, EXL3_VERIFY_NB in kernels/exl3.hip).
@@ -434,19 +471,17 @@ int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, ui
         if (part >> 32) return fail("sz_moe_layer_verify: a projection of 4 GiB or more");
         const std::string k1 = "verify_gate_up_" + tag, k2 = "verify_down_" + tag;
         {
+            const uint32_t gx = c.ff / 128, extra = (carry_groups + gx * zs_gu - 1) / (gx * zs_gu);   // rows of the grid for a riding sum
             const sz_arg a[] = {P(rl), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(u), P(plan), P(s->part.ptr),
-                                U32(c.n_expert), U32(c.top_k), U32(m), U32(c.hidden), U32(c.ff)};
-            if (launch(k1.c_str(), c.ff / 128, 2 * S, zs_gu, 256, 0, stream, a)) return 1;   // 4 waves of one 128-block each: EXL3_GU_WAVES, EXL3_VERIFY_NB
+                                U32(c.n_expert), U32(c.top_k), U32(m), U32(c.hidden), U32(c.ff), P(s->dn.ptr), P(c_plan), P(c_sgl), P(c_y), U32(c_mode)};
+            if (launch(k1.c_str(), gx, 2 * S + extra, zs_gu, 256, 0, stream, a)) return 1;   // 4 waves of one 128-block each: EXL3_GU_WAVES, EXL3_VERIFY_NB
         }
         {
             const sz_arg a[] = {P(rl), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(plan), P(s->part.ptr), P(s->dn.ptr),
                                 U32(c.n_expert), U32(c.top_k), U32(m), U32(c.hidden), U32(c.ff), U32(zs_gu)};
             if (launch(k2.c_str(), c.hidden / 128, S, zs_d, 256, 0, stream, a)) return 1;
         }
-        s->last_fused = true;
-        const sz_arg a[] = {P(s->dn.ptr), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(plan), P(sgl), P(y),
-                            U32(c.top_k), U32(m), U32(c.hidden), U32(c.ff), U32(zs_d == 1 ? 0 : zs_d)};
-        return launch("verify_combine_exl3", c.hidden / 128, m, 1, zs_d == 1 ? 128 : 1024, 0, stream, a);   // zs_d == 1: launch 2 finished the blocks
+        return sum(zs_d, part);
     } else if (!std::getenv("SHADOWZERO_GGUF_PLANNED") && c.ff <= 4096) {
         // the pair form, as the EXL3 layer: routing inside launch 1, SwiGLU inside launch 2, no plan
         const uint32_t S = p.G + m;
@@ -677,7 +712,7 @@ sz_session* sz_session_new(const sz_session_config* cfg) {
     const uint64_t ks_gu = exl3_ksplit(c.hidden), ks_d = exl3_ksplit(c.ff);
     const uint64_t part = std::max<uint64_t>(2ull * p.GT * ks_gu * 4 * c.ff, (uint64_t) p.GT * ks_d * 4 * c.hidden) * 4;
     const uint64_t nparts = c.vocab / 4 + 1;
-    bool bad = s->plan.need(std::max(p.bytes, mma_plan(c.max_rows, c.top_k).bytes)) || s->eg.need(2ull * p.R * c.ff * 4) || s->act.need((uint64_t) p.R * c.ff * 4) ||
+    bool bad = s->plan.need(std::max(p.bytes, mma_plan(c.max_rows, c.top_k).bytes)) || s->plan2.need(std::max(p.bytes, mma_plan(c.max_rows, c.top_k).bytes)) || s->eg.need(2ull * p.R * c.ff * 4) || s->act.need((uint64_t) p.R * c.ff * 4) ||
                s->eo.need((uint64_t) p.R * c.hidden * 4) || s->part.need(part) || s->ids.need(64) ||
                s->dn.need((uint64_t) p.GT * ks_d * 4 * c.hidden * 4);
     if (c.vocab) bad = bad || s->head_part.need(nparts * 4 * 2 * 4);
@@ -833,7 +868,7 @@ int32_t sz_session_set_head_proxy(sz_session* s, uint32_t k_blk) {
 
 uint64_t sz_session_buffer(sz_session* s, int32_t which) {
     if (!s) return 0;
-    const uint64_t at[] = {s->plan.ptr, s->part.ptr, s->dn.ptr, s->eg.ptr, s->eo.ptr, s->hp.w_q2.ptr, s->hp.w_sc.ptr, s->hp.xq.ptr, s->hp.x_sc.ptr,
+    const uint64_t at[] = {s->last_plan ? s->last_plan : s->plan.ptr, s->part.ptr, s->dn.ptr, s->eg.ptr, s->eo.ptr, s->hp.w_q2.ptr, s->hp.w_sc.ptr, s->hp.xq.ptr, s->hp.x_sc.ptr,
                            s->hp.x_corr.ptr, s->hp.bmax.ptr, s->hp.sel.ptr, s->hp.logits.ptr};
     return which >= 0 && which < (int32_t) (sizeof at / sizeof at[0]) ? at[which] : 0;
 }
@@ -869,9 +904,10 @@ int32_t sz_session_last_route(sz_session* s, uint32_t m, uint32_t* idx, float* w
     if (sz_stream_synchronize(stream)) return 1;
     const PlanLayout p = plan_layout(m, s->cfg.top_k);
     const uint64_t n = (uint64_t) m * s->cfg.top_k * 4;
-    if (s->last_fused) return sz_download(idx, s->plan.ptr, n) || sz_download(w, s->plan.ptr + n, n);
-    if (sz_download(idx, s->plan.ptr + p.tidx_off, n)) return 1;
-    return sz_download(w, s->plan.ptr + p.w_off, n);
+    const uint64_t plan = s->last_plan ? s->last_plan : s->plan.ptr;
+    if (s->last_fused) return sz_download(idx, plan, n) || sz_download(w, plan + n, n);
+    if (sz_download(idx, plan + p.tidx_off, n)) return 1;
+    return sz_download(w, plan + p.w_off, n);
 }
 
 int32_t sz_head_argmax(sz_session* s, uint32_t m, uint64_t u, uint64_t ids, uint64_t stream) {
@@ -970,10 +1006,13 @@ int32_t sz_verify_round(sz_session* s, uint32_t m, uint64_t u, uint64_t rl, uint
     if (it == s->graphs.end()) {
         static const bool no_graph = std::getenv("SHADOWZERO_NO_GRAPH") != nullptr;
         auto record = [&]() -> int {
+            // an EXL3 layer's rank-order sum rides the first launch of the layer after it; the last layer's gets its own launch
+            PendingSum ps;
             for (uint32_t l = 0; l < c.n_layers; l++) {
                 const uint64_t off = (uint64_t) l * m;
-                if (moe_layer(s, l, m, u + off * c.hidden * 4, rl + off * c.n_expert * 4, sgl + off * 4, y + off * c.hidden * 4, stream)) return 1;
+                if (moe_layer(s, l, m, u + off * c.hidden * 4, rl + off * c.n_expert * 4, sgl + off * 4, y + off * c.hidden * 4, stream, &ps)) return 1;
             }
+            if (launch_pending_sum(s, ps, m, stream)) return 1;
             if (head_argmax(s, m, head_u, out + 8, stream)) return 1;
             const sz_arg a[] = {P(out + 8), P(drafts), U32(m - 1), P(out)};
             return launch("verify_accept", 1, 1, 1, 64, 0, stream, a);

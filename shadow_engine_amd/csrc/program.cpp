@@ -269,8 +269,8 @@ int launch(const char* name, uint32_t gx, uint32_t gy, uint32_t gz, uint32_t bx,
         }
         fn = it->second;
     }
-    uint64_t vals[16];
-    void* ptrs[16];
+    uint64_t vals[24];
+    void* ptrs[24];
     for (int i = 0; i < nargs; i++) {
         vals[i] = args[i].value;   // little-endian: a 4-byte parameter reads the low half of its slot
         ptrs[i] = &vals[i];

@@ -95,7 +95,7 @@ struct SzEntry {
     const char* name;
     int file;
     int nparams;
-    int kinds[16];
+    int kinds[24];
 };
 int entry_count();
 const SzEntry* entry(int i);

@@ -471,6 +471,34 @@ extern "C" __global__ void __launch_bounds__(64) exl3_finish_rows(const float* p
 // between a routing result and the first request for that expert's weights.
 // pbuf holds u32 tidx[m k] | f32 w[m k] | u32 cnt[m].
 
+// The rank-order sum of token j's finished down products for the 128 columns of block ob (launch 2 has finished every
+// pair's block: no split over its inputs), column ob * 128 + tid for tid < 128: y[j] = sum over the cnt[j] experts of
+// w[j, t] * dn[j k + t] + sigmoid(gl[j]) * dn[m k + j] (moe_combine_qwen_rows, kernels/forward.cu:2568).  Every load goes
+// out before the first is waited for.  pbuf = u32 tidx[m k] | f32 w[m k] | u32 cnt[m].
+__device__ __forceinline__ void exl3_combine_finished(const float* __restrict__ dn, const u8* __restrict__ pbuf, const float* __restrict__ gl,
+                                                      float* __restrict__ y, u32 k, u32 m, u32 hidden, bool shared, u32 ob, u32 j, u32 tid) {
+    const u32 G = m * k;
+    const float* wts = (const float*) (pbuf + G * 4);
+    const u32* cnt = (const u32*) (pbuf + 2 * G * 4);
+    const u32 col = ob * 128 + tid;
+    float v[17], w[16];
+#pragma unroll
+    for (int i = 0; i < 16; i++) {
+        const u32 pair = j * k + min((u32) i, k - 1);
+        v[i] = dn[(u64) pair * hidden + col];
+        w[i] = wts[pair];
+    }
+    v[16] = shared ? dn[(u64) (G + j) * hidden + col] : 0.0f;
+    const float sg = shared ? sigmoidf_ref(gl[j]) : 0.0f;
+    const u32 c = cnt[j];
+    float a = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 16; i++)
+        if ((u32) i < c) a += w[i] * v[i];
+    if (shared) a += sg * v[16];
+    y[(u64) j * hidden + col] = a;
+}
+
 // Launch 1's workgroup: EXL3_GU_WAVES waves, each takes EXL3_VERIFY_NB consecutive 128-blocks of the input through a ring
 // of EXL3_GU_DEPTH rows (grid z = ceil(hidden / 128 / (waves * blocks))).  One block a wave with a 4-row ring puts twice as
 // many waves on a SIMD as two blocks a wave with an 8-row ring, for the same LDS: the waves spend most of their life
@@ -484,11 +512,21 @@ extern "C" __global__ void __launch_bounds__(64) exl3_finish_rows(const float* p
 // Launch 1: routing (every workgroup of a routed pair redoes its token's selection on one of its waves; the workgroups
 // with blockIdx.x == 0 and blockIdx.z == 0 of the gate half also publish tidx) and the gate and up products' partial
 // sums: gup[((sel * S + pair) * zs + z)][ff], S = m (k + 1), sel 0 = gate, 1 = up, zs = gridDim.z.
-// grid = (ff / 128, 2 S, zs), block 64 * EXL3_GU_WAVES.
+// grid = (ff / 128, 2 S + c, zs), block 64 * EXL3_GU_WAVES; c = 0, or the rows that give (hidden / 128) m more workgroups
+// for the sum of the layer before (cmode).
 template <int K, bool H = false>
 __device__ __forceinline__ void verify_gate_up_kernel(const float* __restrict__ logits, u64 ebase, u64 estride, u64 shbase, u32 part,
                                                       const float* __restrict__ u, u8* __restrict__ pbuf, float* __restrict__ gup, u32 ne, u32 k,
-                                                      u32 m, u32 hidden, u32 ff) {
+                                                      u32 m, u32 hidden, u32 ff, const float* __restrict__ cdn, const u8* __restrict__ cpbuf,
+                                                      const float* __restrict__ cgl, float* __restrict__ cy, u32 cmode) {
+    if (blockIdx.y >= 2 * (m * k + m)) {
+        // rows of the grid past the pairs (cmode != 0): the rank-order sum of the layer before this one, whose launch 3 rides
+        // here (same batch and shapes; cdn its finished down products, cpbuf its routing, cgl its shared gate logits, cy its
+        // output; cmode 2: it has a shared expert), a workgroup a (token, 128-column block)
+        const u32 ci = ((blockIdx.y - 2 * (m * k + m)) * gridDim.z + blockIdx.z) * gridDim.x + blockIdx.x, nb = hidden / 128;
+        if (cmode && ci < nb * m && threadIdx.x < 128) exl3_combine_finished(cdn, cpbuf, cgl, cy, k, m, hidden, cmode == 2, ci % nb, ci / nb, threadIdx.x);
+        return;
+    }
     constexpr int NB = EXL3_VERIFY_NB, WA = EXL3_GU_WAVES, D = EXL3_GU_DEPTH;
     __shared__ __attribute__((aligned(16))) u32 wb_all[WA][Exl3Rows<K, D, H>::words];   // the waves' trellis rows; before that, the routing's scratch
     __shared__ float xw_all[WA][NB * 128];
@@ -697,8 +735,9 @@ __device__ __forceinline__ void verify_down_kernel(const float* __restrict__ log
 #define EXL3_VERIFY_ENTRIES(K)                                                                                                            \
     extern "C" __global__ void __launch_bounds__(64 * EXL3_GU_WAVES, EXL3_GU_OCC(K)) verify_gate_up_exl3_##K(const float* logits, u64 ebase, u64 estride, u64 shbase, u32 part, \
                                                                                   const float* u, u8* pbuf, float* gup, u32 ne, u32 k, u32 m, \
-                                                                                  u32 hidden, u32 ff) {                                       \
-        verify_gate_up_kernel<K>(logits, ebase, estride, shbase, part, u, pbuf, gup, ne, k, m, hidden, ff);                               \
+                                                                                  u32 hidden, u32 ff, const float* cdn, const u8* cpbuf,      \
+                                                                                  const float* cgl, float* cy, u32 cmode) {                   \
+        verify_gate_up_kernel<K>(logits, ebase, estride, shbase, part, u, pbuf, gup, ne, k, m, hidden, ff, cdn, cpbuf, cgl, cy, cmode);   \
     }                                                                                                                                     \
     extern "C" __global__ void __launch_bounds__(256, EXL3_VERIFY_WAVES(K)) verify_down_exl3_##K(const float* logits, u64 ebase, u64 estride, u64 shbase, u32 part,   \
                                                                                u8* pbuf, const float* gup, float* dn, u32 ne, u32 k, u32 m,   \
@@ -710,8 +749,9 @@ __device__ __forceinline__ void verify_down_kernel(const float* __restrict__ log
 #define EXL3_VERIFY_HALF_ENTRIES(K)                                                                                                       \
     extern "C" __global__ void __launch_bounds__(64 * EXL3_GU_WAVES, EXL3_GU_OCC(K + 1)) verify_gate_up_exl3h_##K(const float* logits, u64 ebase, u64 estride, u64 shbase, u32 part, \
                                                                                   const float* u, u8* pbuf, float* gup, u32 ne, u32 k, u32 m, \
-                                                                                  u32 hidden, u32 ff) {                                       \
-        verify_gate_up_kernel<K, true>(logits, ebase, estride, shbase, part, u, pbuf, gup, ne, k, m, hidden, ff);                         \
+                                                                                  u32 hidden, u32 ff, const float* cdn, const u8* cpbuf,      \
+                                                                                  const float* cgl, float* cy, u32 cmode) {                   \
+        verify_gate_up_kernel<K, true>(logits, ebase, estride, shbase, part, u, pbuf, gup, ne, k, m, hidden, ff, cdn, cpbuf, cgl, cy, cmode); \
     }                                                                                                                                     \
     extern "C" __global__ void __launch_bounds__(256, EXL3_VERIFY_WAVES(K + 1)) verify_down_exl3h_##K(const float* logits, u64 ebase, u64 estride, u64 shbase, u32 part, \
                                                                                u8* pbuf, const float* gup, float* dn, u32 ne, u32 k, u32 m,   \
@@ -746,26 +786,7 @@ extern "C" __global__ void __launch_bounds__(1024) verify_combine_exl3(const flo
     const float* wts = (const float*) (pbuf + G * 4);
     const u32* cnt = (const u32*) (pbuf + 2 * G * 4);
     if (zs == 0) {
-        // launch 2 has finished every pair's block already (no split over its inputs): weight and add, in rank order.  Every
-        // load goes out before the first is waited for.
-        if (t >= 2) return;
-        const u32 col = ob * 128 + threadIdx.x;
-        float v[17], w[16];
-#pragma unroll
-        for (int i = 0; i < 16; i++) {
-            const u32 pair = j * k + min((u32) i, k - 1);
-            v[i] = dn[(u64) pair * hidden + col];
-            w[i] = wts[pair];
-        }
-        v[16] = shbase ? dn[(u64) (G + j) * hidden + col] : 0.0f;
-        const float sg = shbase ? sigmoidf_ref(gl[j]) : 0.0f;
-        const u32 c = cnt[j];
-        float a = 0.0f;
-#pragma unroll
-        for (int i = 0; i < 16; i++)
-            if ((u32) i < c) a += w[i] * v[i];
-        if (shbase) a += sg * v[16];
-        y[(u64) j * hidden + col] = a;
+        if (t < 2) exl3_combine_finished(dn, pbuf, gl, y, k, m, hidden, shbase != 0, ob, j, threadIdx.x);
         return;
     }
     const u32 c = cnt[j];
@@ -1223,11 +1244,19 @@ extern "C" __global__ void __launch_bounds__(64) cols_plan(u64* wtab, u32* gtab,
 // 8 bytes, their pair numbers as 8 u16 (pair j k + t of token j and rank t, m k + j for the shared expert: the row of the
 // partial sums and of launch 2's output, which verify_combine_exl3 reads as it does after the exact launches).
 
-// grid 1, block 64 m.  Wave j selects token j's experts (lane t < k then holds rank t's); the items come out of three tables
+// grid 1 (+ the workgroups of a riding sum), block 64 m.  Wave j selects token j's experts (lane t < k then holds rank t's); the items come out of three tables
 // in LDS indexed by expert: the lowest pair that chose it (that pair's thread writes the item), the tokens that chose it as
 // a bit mask, and each such token's rank.  The routing weights are not needed before launch 3 and are left to a spare
 // workgroup of launch 1 (verify_route_weights below).
-extern "C" __global__ void __launch_bounds__(512) verify_plan_exl3(const float* logits, u8* pbuf, u32 ioff, u32 ne, u32 k, u32 m, u32 shared) {
+// Workgroups 1 .. (hidden / 128) m (cmode != 0): the rank-order sum of the layer before, as in verify_gate_up_kernel.
+extern "C" __global__ void __launch_bounds__(512) verify_plan_exl3(const float* logits, u8* pbuf, u32 ioff, u32 ne, u32 k, u32 m, u32 shared, u32 hidden,
+                                                                   const float* cdn, const u8* cpbuf, const float* cgl, float* cy, u32 cmode) {
+    if (blockIdx.x > 0) {
+        const u32 ci = blockIdx.x - 1, nb = hidden / 128;
+        if (cmode && ci < nb * m)
+            for (u32 t = threadIdx.x; t < 128; t += blockDim.x) exl3_combine_finished(cdn, cpbuf, cgl, cy, k, m, hidden, cmode == 2, ci % nb, ci / nb, t);
+        return;
+    }
     __shared__ double ex[8 * 512];   // the exact selection's scratch, a wave's 512 doubles
     __shared__ u32 top[8][16];
     __shared__ u32 lowest[512];      // expert -> the lowest pair number that chose it
