@@ -44,7 +44,7 @@ SIMDS = 256 * 4                                  # 256 compute units x 4 SIMDs; 
 
 
 def load_counters(sz):
-    """profiles/counters.json (written by `python -m shadow_engine_amd.profile_counters` from rocprofv3 databases): per-kernel
+    """profiles/counters.json (written by `python3 profile_counters.py` from rocprofv3 databases): per-kernel
     hardware counters of the benchmark's workloads, stamped with the cache keys of the kernel files they were measured on.
     Returns (counters or None, stale): stale maps every kernel whose file has changed since (or every kernel, when the
     file is missing) to the reason its counters are not quoted."""

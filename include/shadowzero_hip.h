@@ -157,6 +157,10 @@ int32_t sz_session_set_layer(sz_session*, uint32_t layer, int32_t expert_type, u
  * multiples of 128; the head of an EXL3 checkpoint, session.rs:7179-7187).  The fused arg-max (sz_head_argmax,
  * sz_verify_round) exists for Q8_0 and EXL3; logits and the top 64 for all three. */
 int32_t sz_session_set_head(sz_session*, int32_t ggml_type, uint64_t w);
+/* LDS a workgroup of the EXL3 head's kernel takes for m rows (0 for another type): the head entry points refuse a call
+ * whose need is above a compute unit's 160 KiB (hidden 4096 takes all 8 rows at any rate, hidden 8192 up to 4), and
+ * sz_session_set_head a head that cannot take one row.  No counterpart in the reference (its kernels take 64 rows in registers). */
+uint32_t sz_exl3_head_lds_bytes(int32_t type, uint32_t hidden, uint32_t m);
 /* The optional, INEXACT 2-bit screen of an EXL3 head for the top-64 hand-off (HeadProxy, session.rs:428-441, built at
  * session.rs:2631-2674 by exl3_build_q2_proxy_K, kernels/exl3.cu:916-996; used by head_top_at, session.rs:5952-6022): off by
  * default and after every sz_session_set_head, as the reference's exact mode has it (session.rs:786).  k_blk > 0 builds the
@@ -209,37 +213,6 @@ int32_t sz_verify_accept(const uint32_t* ids, const uint32_t* drafts, uint32_t n
 int32_t sz_lookup_draft(const uint32_t* hist, uint64_t n_hist, uint32_t k, const uint32_t* lens, uint32_t n_lens, uint32_t* drafts,
                         uint32_t* n_drafts);
 
-/* ---- the drafters that need no second model, and the policy that picks a round's window (host code; (f) of the path's callers) --
- * The suffix drafter (crates/shadowzero-serve/src/engine.rs:844-1015 SuffixDrafter): every trigram of the pushed tokens
- * remembers the last four places it ended.  propose: among those places for the trigram the sequence ends in, the one whose
- * match backwards is longest (at most max_match tokens, the more recent on a tie, at least min_match: 0 = the drafter's own,
- * never under 3); the up to max_k tokens that followed it are the draft.  `extra` (n_extra may be 0) is a neural drafter's
- * proposal that goes behind the history for the question only (propose_after, engine.rs:998): the index keeps what was pushed. */
-typedef struct sz_suffix_drafter sz_suffix_drafter;
-sz_suffix_drafter* sz_suffix_drafter_new(uint32_t min_match, uint32_t max_match, uint32_t capacity_tokens);
-void sz_suffix_drafter_free(sz_suffix_drafter*);
-int32_t sz_suffix_drafter_extend(sz_suffix_drafter*, const uint32_t* tokens, uint32_t n);          /* push / extend, engine.rs:929-951 */
-uint64_t sz_suffix_drafter_len(const sz_suffix_drafter*);
-int32_t sz_suffix_drafter_propose(sz_suffix_drafter*, const uint32_t* extra, uint32_t n_extra, uint32_t max_k, uint32_t min_match,
-                                  uint32_t* drafts, uint32_t* n_drafts, uint32_t* match_len);
-/* The draft policy (engine.rs:1017-1311 DraftPolicy): running means of a round's cost by its number of rows t (1 + drafts,
- * at most 8) and of the tokens a neural window yields, decayed counts of kept and refused looked-up drafts by match length.
- *   neural_k      how many drafts to ask the neural drafter for (base_spec, one more after full windows, 2 after empty ones)
- *   choose        neural window of t_neural rows, or a lookup window (*lookup = 1) of *t rows out of lookup_k available drafts
- *   chain         how many of k_avail looked-up tokens to put behind a neural window whose drafts all hold with p_neural
- *   observe       what a round did: lookup or neural, its rows t, accepted drafts, the lookup's match length, its time
- *   observe_chain the same for a chained round (t_neural rows of the neural window, then k_chain looked-up tokens) */
-typedef struct sz_draft_policy sz_draft_policy;
-sz_draft_policy* sz_draft_policy_new(uint32_t max_t, uint32_t base_spec, double margin);
-void sz_draft_policy_free(sz_draft_policy*);
-uint32_t sz_draft_policy_neural_k(const sz_draft_policy*, uint32_t rem_tokens);
-int32_t sz_draft_policy_choose(const sz_draft_policy*, uint32_t t_neural, uint32_t lookup_k, uint32_t match_len, int32_t* lookup, uint32_t* t);
-uint32_t sz_draft_policy_chain(const sz_draft_policy*, uint32_t t_neural, double p_neural, uint32_t k_avail, uint32_t match_len);
-int32_t sz_draft_policy_observe(sz_draft_policy*, int32_t lookup, uint32_t t, uint32_t accepted, uint32_t match_len, double round_ms);
-int32_t sz_draft_policy_observe_chain(sz_draft_policy*, uint32_t t_neural, uint32_t k_chain, uint32_t accepted, uint32_t match_len, double round_ms);
-/* For tests and logs: the running acceptance, the rounds seen, cost_ms(t) for t = 1..8, and the kept-rate of looked-up and of
- * chained drafts for the four match-length classes (any pointer may be null). */
-int32_t sz_draft_policy_state(const sz_draft_policy*, double* accept_ema, double* rounds, double* cost_ms8, double* lookup_rate4, double* chain_rate4);
 /* ---- the rollback point of a speculative pass: device state saved and put back, one launch each way.
  * The reference keeps the recurrent layers' states of a session in a device-side snapshot that it takes again before
  * every pass (GpuSession::snapshot_again, crates/shadowzero-cuda/src/session.rs:3407-3452) and restores when drafts are

@@ -17,7 +17,7 @@ workload of bench.py, ARGS its flags (`--workload W`, nothing for the default on
 
 then, in the same session (the databases are large and are not kept):
 
-    python3 -m shadow_engine_amd.profile_counters PROF
+    python3 profile_counters.py PROF
 
 A workload may have any subset of the passes.  Memory counters are scaled by what the same counter reads for the plain
 copy of known size that `--copy-calibration` appends to the run (copy_words16: 1 GiB read, 1 GiB written).
@@ -27,7 +27,7 @@ import os
 import sqlite3
 import sys
 
-ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ROOT = os.path.dirname(os.path.abspath(__file__))
 OURS = ("verify_", "decode_", "head_", "argmax_merge", "copy_", "matvec_", "route_", "swiglu", "moe_", "prefill_", "quant_act", "scatter_", "exl3_", "topk_", "proxy_")
 NAMES = {"config5": ("verify_round_config5", "the default benchmark workload (config 5: 48-layer verify round on a 4-row batch, mixed EXL3 K in {2,3,4}, Q8_0 lm_head)", ""),
          "config3": ("verify_layer_and_head_config3", "bench.py --workload config3 (one EXL3 K=3 MoE layer for 4 tokens + Q8_0 head + acceptance)", " --workload config3"),
@@ -72,7 +72,7 @@ def trace_summary(d, plain, title, args):
     tot = sum(x[2] for x in r) or 1
     out = ["Kernel trace of %s on one MI355X." % title,
            "Command (from the repository root after cd /tmp && export TMPDIR=/tmp && cd <repo>; the rocpd database it writes is summarised by",
-           "python3 -m shadow_engine_amd.profile_counters with: select name, count(*), sum(duration), avg, min, max from kernels group by name):",
+           "python3 profile_counters.py with: select name, count(*), sum(duration), avg, min, max from kernels group by name):",
            "  rocprofv3 --kernel-trace --stats -d %s/W/trace -o run -- python3 bench.py%s --steps 20 --warmup 3%s" % (PROF, args, TAIL), "",
            "%-28s %7s %12s %10s %10s %10s %7s" % ("kernel (this library's only)", "calls", "total_us", "avg_us", "min_us", "max_us", "pct")]
     for n, c, t, a, mn, mx in r:
@@ -188,7 +188,7 @@ def main(prof, out_dir):
     import shadow_engine_amd as sz
     PROF = prof.rstrip("/")
     os.makedirs(out_dir, exist_ok=True)
-    counters = {"kernel_keys": sz.program_keys(), "made_by": "python3 -m shadow_engine_amd.profile_counters (commands in its docstring and in profiles/*.txt)",
+    counters = {"kernel_keys": sz.program_keys(), "made_by": "python3 profile_counters.py (commands in its docstring and in profiles/*.txt)",
                 "peaks": {"simds": SIMDS, "cycles_per_wave64_vector_instruction": 4}, "workloads": {}}
     try:
         # workloads summarised earlier on the same kernel sources stay; a file of other sources is started afresh

@@ -147,6 +147,7 @@ _SIGNATURES = {
     "sz_session_set_head_proxy": (_i32, [_vp, _u32]),
     "sz_session_set_graph": (_i32, [_vp, _i32]),
     "sz_session_set_expert_mode": (_i32, [_vp, _i32]),
+    "sz_exl3_head_lds_bytes": (_u32, [_i32, _u32, _u32]),
     "sz_moe_layer_verify": (_i32, [_vp, _u32, _u32, _u64, _u64, _u64, _u64, _u64]),
     "sz_session_set_router": (_i32, [_vp, _u32, _i32, _u64, _i32, _u64]),
     "sz_moe_router_verify": (_i32, [_vp, _u32, _u32, _u64, _u64]),
@@ -164,19 +165,6 @@ _SIGNATURES = {
     "sz_verify_accept": (_i32, [_vp, _vp, _u32, C.POINTER(_u32)]),
     "sz_verify_round": (_i32, [_vp, _u32, _u64, _u64, _u64, _u64, _u64, _u64, _u64, _u64]),
     "sz_lookup_draft": (_i32, [_vp, _u64, _u32, _vp, _u32, _vp, C.POINTER(_u32)]),
-    "sz_suffix_drafter_new": (_vp, [_u32, _u32, _u32]),
-    "sz_suffix_drafter_free": (None, [_vp]),
-    "sz_suffix_drafter_extend": (_i32, [_vp, _vp, _u32]),
-    "sz_suffix_drafter_len": (_u64, [_vp]),
-    "sz_suffix_drafter_propose": (_i32, [_vp, _vp, _u32, _u32, _u32, _vp, C.POINTER(_u32), C.POINTER(_u32)]),
-    "sz_draft_policy_new": (_vp, [_u32, _u32, C.c_double]),
-    "sz_draft_policy_free": (None, [_vp]),
-    "sz_draft_policy_neural_k": (_u32, [_vp, _u32]),
-    "sz_draft_policy_choose": (_i32, [_vp, _u32, _u32, _u32, C.POINTER(_i32), C.POINTER(_u32)]),
-    "sz_draft_policy_chain": (_u32, [_vp, _u32, C.c_double, _u32, _u32]),
-    "sz_draft_policy_observe": (_i32, [_vp, _i32, _u32, _u32, _u32, C.c_double]),
-    "sz_draft_policy_observe_chain": (_i32, [_vp, _u32, _u32, _u32, _u32, C.c_double]),
-    "sz_draft_policy_state": (_i32, [_vp, _vp, _vp, _vp, _vp, _vp]),
     "sz_snapshot_new": (_i32, [_vp, _vp, _u32, C.POINTER(_vp)]),
     "sz_snapshot_free": (None, [_vp]),
     "sz_snapshot_bytes": (_u64, [_vp]),
@@ -616,74 +604,6 @@ def lookup_draft(hist, k, lens=(3, 2)):
     out, n = np.zeros(max(k, 1), np.uint32), _u32()
     check(lib().sz_lookup_draft(h.ctypes.data, h.size, k, ln.ctypes.data, ln.size, out.ctypes.data, C.byref(n)))
     return out[:n.value].tolist()
-
-
-class SuffixDrafter:
-    """The trigram suffix drafter (engine.rs:844-1015): extend() with what was said, propose() a continuation of the longest
-    earlier occurrence of the tail, propose_after(extra) the same behind a neural drafter's proposal."""
-
-    def __init__(self, min_match, max_match, capacity_tokens=4096):
-        self._h = lib().sz_suffix_drafter_new(min_match, max_match, capacity_tokens)
-
-    def extend(self, tokens):
-        t = np.ascontiguousarray(tokens, np.uint32)
-        check(lib().sz_suffix_drafter_extend(self._h, t.ctypes.data, t.size))
-
-    def __len__(self):
-        return int(lib().sz_suffix_drafter_len(self._h))
-
-    def propose(self, max_k, min_match=0, extra=()):
-        """(drafts, match length)"""
-        e = np.ascontiguousarray(extra, np.uint32)
-        out, n, ml = np.zeros(max(max_k, 1), np.uint32), _u32(), _u32()
-        check(lib().sz_suffix_drafter_propose(self._h, e.ctypes.data, e.size, max_k, min_match, out.ctypes.data, C.byref(n), C.byref(ml)))
-        return out[:n.value].tolist(), ml.value
-
-    def propose_after(self, extra, max_k):
-        return self.propose(max_k, 0, extra)
-
-    def __del__(self):
-        try:
-            lib().sz_suffix_drafter_free(self._h)
-        except Exception:
-            pass
-
-
-class DraftPolicy:
-    """The window policy of a speculative round (engine.rs:1017-1311)."""
-
-    def __init__(self, max_t, base_spec, margin):
-        self._h = lib().sz_draft_policy_new(max_t, base_spec, margin)
-
-    def neural_k(self, rem_tokens):
-        return int(lib().sz_draft_policy_neural_k(self._h, rem_tokens))
-
-    def choose(self, t_neural, lookup_k, match_len):
-        """(lookup?, rows of the window)"""
-        lk, t = _i32(), _u32()
-        check(lib().sz_draft_policy_choose(self._h, t_neural, lookup_k, match_len, C.byref(lk), C.byref(t)))
-        return bool(lk.value), t.value
-
-    def chain(self, t_neural, p_neural, k_avail, match_len):
-        return int(lib().sz_draft_policy_chain(self._h, t_neural, p_neural, k_avail, match_len))
-
-    def observe(self, lookup, t, accepted, match_len, round_ms):
-        check(lib().sz_draft_policy_observe(self._h, int(bool(lookup)), t, accepted, match_len, round_ms))
-
-    def observe_chain(self, t_neural, k_chain, accepted, match_len, round_ms):
-        check(lib().sz_draft_policy_observe_chain(self._h, t_neural, k_chain, accepted, match_len, round_ms))
-
-    def state(self):
-        ema, rounds = C.c_double(), C.c_double()
-        cost, lr, cr = np.zeros(8), np.zeros(4), np.zeros(4)
-        check(lib().sz_draft_policy_state(self._h, C.addressof(ema), C.addressof(rounds), cost.ctypes.data, lr.ctypes.data, cr.ctypes.data))
-        return {"accept_ema": ema.value, "rounds": rounds.value, "cost_ms": cost, "lookup_rate": lr, "chain_rate": cr}
-
-    def __del__(self):
-        try:
-            lib().sz_draft_policy_free(self._h)
-        except Exception:
-            pass
 
 
 class Snapshot:

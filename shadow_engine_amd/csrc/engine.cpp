@@ -599,14 +599,29 @@ int head_argmax_mfma(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uin
     return launch("argmax_merge_parts", m, 1, 1, 256, 0, stream, b);
 }
 
+bool head_is_exl3(const sz_session* s) { return s->head_type >= 1021 && s->head_type <= 1028; }
+
+// LDS of a workgroup of head_exl3_K for m rows: the four waves' 4-row rings (static; a row is 64 lanes x 4 words at K = 3 and
+// 4, x K words otherwise) and the A rows, 4 KiB for every 512 inputs and every two rows (dynamic).  A compute unit of the
+// MI355X has 160 KiB.
+const uint32_t CU_LDS_BYTES = 160 * 1024;
+uint32_t exl3_head_lds_dynamic(uint32_t hidden, uint32_t m) { return 4 * ((hidden / 128 + 3) / 4) * ((m + 1) / 2) * 1024; }
+uint32_t exl3_head_lds(uint32_t bits, uint32_t hidden, uint32_t m) {
+    const uint32_t stride = (bits == 3 || bits == 4) ? 4 : bits;
+    return 4 * (4 * 64 * stride) * 4 + exl3_head_lds_dynamic(hidden, m);
+}
+
 int head_check(sz_session* s, uint32_t m, uint64_t u, const char* who) {
     if (!s->head_w) return fail(std::string(who) + ": no head set");
     if (m == 0 || m > s->cfg.max_rows) return fail(std::string(who) + ": " + std::to_string(m) + " rows");
     if (u & 15) return fail(std::string(who) + ": activations must be 16-byte aligned");
+    if (head_is_exl3(s) && exl3_head_lds((uint32_t) s->head_type - 1020, s->cfg.hidden, m) > CU_LDS_BYTES)
+        return fail(std::string(who) + ": an EXL3 head of hidden " + std::to_string(s->cfg.hidden) + " at " + std::to_string(s->head_type - 1020) + " bits takes " +
+                    std::to_string(exl3_head_lds((uint32_t) s->head_type - 1020, s->cfg.hidden, m)) + " bytes of LDS for " + std::to_string(m) +
+                    " rows, a compute unit has " + std::to_string(CU_LDS_BYTES) + ": fewer rows a call");
     return 0;
 }
 
-bool head_is_exl3(const sz_session* s) { return s->head_type >= 1021 && s->head_type <= 1028; }
 bool head_argmax_supported(const sz_session* s) { return s->head_type == SZ_TYPE_Q8_0 || head_is_exl3(s); }
 
 // An EXL3 head (kernels/exl3.cu:349-461, 610-625 of the reference: rotate the rows once, then one pass over the matrix for all
@@ -618,7 +633,7 @@ int head_exl3(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uint64_t i
         const sz_arg a[] = {P(s->head_w), P(u), U32(c.hidden), P(s->head_xa.ptr), P(s->head_inv.ptr), U32(c.hidden)};
         if (launch("exl3_head_rotate", m, 1, 1, 64 * std::min<uint32_t>(16, kbs), 0, stream, a)) return 1;
     }
-    const uint32_t nparts = c.vocab / 128, lds = 4 * ((kbs + 3) / 4) * ((m + 1) / 2) * 1024;
+    const uint32_t nparts = c.vocab / 128, lds = exl3_head_lds_dynamic(c.hidden, m);
     const std::string kn = "head_exl3_" + std::to_string(bits);
     const sz_arg a[] = {P(s->head_w), P(s->head_xa.ptr), P(s->head_inv.ptr), P(logits), U32(c.vocab), P(s->head_part.ptr), U32(c.hidden), U32(c.vocab), U32(m), P(0)};
     if (launch(kn.c_str(), nparts, 1, 1, 256, lds, stream, a)) return 1;
@@ -662,7 +677,7 @@ int head_proxy_sparse(sz_session* s, uint32_t m, uint64_t u, uint32_t need_k, ui
         const sz_arg a[] = {P(s->hp.seen.ptr), U32(n_ob), U32(max_sel), P(s->hp.sel.ptr)};
         if (launch("proxy_compact_seen", 1, 1, 1, 64, 0, stream, a)) return 1;
     }
-    const uint32_t lds = 4 * ((kbs + 3) / 4) * ((m + 1) / 2) * 1024;
+    const uint32_t lds = exl3_head_lds_dynamic(c.hidden, m);
     const std::string kn = "head_exl3_" + std::to_string(bits);
     const sz_arg a[] = {P(s->head_w), P(s->head_xa.ptr), P(s->head_inv.ptr), P(s->hp.logits.ptr), U32(max_sel * 128), P(s->head_part.ptr),
                         U32(c.hidden), U32(c.vocab), U32(m), P(s->hp.sel.ptr)};
@@ -826,6 +841,9 @@ int32_t sz_session_set_head(sz_session* s, int32_t ty, uint64_t w) {
     if (exl3) {
         const sz_session_config& c = s->cfg;
         if (c.vocab == 0 || c.vocab % 128 || c.hidden % 128 || c.hidden > 8192) return fail("sz_session_set_head: an EXL3 head needs hidden (<= 8192) and the vocabulary to be multiples of 128");
+        // a head that cannot take even one row is refused here; how many rows a call may bring is checked call by call
+        if (exl3_head_lds((uint32_t) ty - 1020, c.hidden, 1) > CU_LDS_BYTES)
+            return fail("sz_session_set_head: an EXL3 head of hidden " + std::to_string(c.hidden) + " does not fit a compute unit's LDS");
         if (s->head_xa.need((uint64_t) c.hidden / 128 * 16 * 256) || s->head_inv.need(64)) return 1;
     }
     s->head_type = ty;
@@ -834,6 +852,10 @@ int32_t sz_session_set_head(sz_session* s, int32_t ty, uint64_t w) {
     for (auto& g : s->graphs) sz_graph_destroy(g.second);
     s->graphs.clear();
     return 0;
+}
+
+uint32_t sz_exl3_head_lds_bytes(int32_t ty, uint32_t hidden, uint32_t m) {
+    return (ty >= 1021 && ty <= 1028) ? exl3_head_lds((uint32_t) ty - 1020, hidden, m) : 0;
 }
 
 int32_t sz_session_set_head_proxy(sz_session* s, uint32_t k_blk) {

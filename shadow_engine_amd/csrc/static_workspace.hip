@@ -12,6 +12,7 @@
 // library (csrc/hipbind.cpp) that pass them to the libamdhip64 bound at run time.
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <string>
 
 #include "shadowzero_hip.h"
@@ -29,17 +30,19 @@ int static_workspace_setup(int device);
 static __device__ __align__(256) unsigned char scratch[SZ_STATIC_WORKSPACE_BYTES];
 
 enum { SZ_MAX_DEVICES = 64 };
-static void* g_workspace[SZ_MAX_DEVICES];   // the array's device address on each GPU that has been set up
+// the array's device address on each GPU that has been set up; sz_init and the entry point may look it up from different
+// host threads at the same time (both find the same address), hence atomic
+static std::atomic<void*> g_workspace[SZ_MAX_DEVICES];
 
 // Called by sz_init with `device` current (and by the entry point for a device it has not seen).
 int sz::static_workspace_setup(int device) {
     if (device < 0 || device >= SZ_MAX_DEVICES) return fail("static workspace: device " + std::to_string(device) + " is out of range");
-    if (g_workspace[device]) return 0;
+    if (g_workspace[device].load(std::memory_order_acquire)) return 0;
     void* ptr = nullptr;
     const hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
     if (e != hipSuccess || !ptr)
         return fail("hipGetSymbolAddress(static workspace) on device " + std::to_string(device) + ": code " + std::to_string((int) e));
-    g_workspace[device] = ptr;
+    g_workspace[device].store(ptr, std::memory_order_release);
     return 0;
 }
 
@@ -57,5 +60,5 @@ extern "C" int32_t sz_matvec_cols_static(int32_t ggml_type, uint64_t w, uint64_t
                         std::to_string((uint64_t) SZ_STATIC_WORKSPACE_BYTES) + "; use sz_matvec_cols with a workspace of the caller's");
     // nothing in the workspace has to start at zero: the plan launch writes every table entry it reads and the partial sums
     // are all written before the finishing launch adds them, so the last call's contents are simply overwritten
-    return sz::matvec_cols_dev(ggml_type, w, cols, rows, x, xs, y, ys, m, (uint64_t) g_workspace[device], SZ_STATIC_WORKSPACE_BYTES, stream);
+    return sz::matvec_cols_dev(ggml_type, w, cols, rows, x, xs, y, ys, m, (uint64_t) g_workspace[device].load(std::memory_order_acquire), SZ_STATIC_WORKSPACE_BYTES, stream);
 }

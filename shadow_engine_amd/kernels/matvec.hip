@@ -599,7 +599,8 @@ __device__ __forceinline__ void verify_down_gguf(const float* logits, u64 ebase,
 // itself, and the combine launch goes away.  Launch 1 then hands over act = silu(gate) * up instead of the two sums (a
 // workgroup takes the same rows of gate and of up), and one wave of it computes the routing weights, which launch 2 only reads.
 // pbuf as above; act holds S rows of ff floats.  The sums are rows_body's single-input sums and the combine is
-// moe_combine_qwen_rows's arithmetic, so y has the bits of the three-launch form.
+// moe_combine_qwen_rows's arithmetic; the routing weights are ex_t over the sum of the chosen ex (route_weights_chosen), within
+// a unit in the last place of the three-launch form's, so y agrees with that form to the last bit or two, not bit for bit.
 
 // floor(x / d) for x < 65536 by one multiplication: `magic` = fast_div_magic(d), 1 <= d < 65536 (the one division, done once).
 __device__ __forceinline__ u32 fast_div_magic(u32 d) { return 0xffffffffu / d + 1u; }

@@ -436,28 +436,26 @@ extern "C" __global__ void __launch_bounds__(1024) proxy_pick_rows(const float* 
     const u32 tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
     const float* row = bmax + (u64) blockIdx.x * n_ob;
     if (tid < 256) {
-        float lv[4] = {-3.0e38f, -3.0e38f, -3.0e38f, -3.0e38f};
-        u32 li[4] = {0xffffffffu, 0xffffffffu, 0xffffffffu, 0xffffffffu};
+        // the thread's four best as sorted keys (value descending, block ascending, as the rest of the kernel orders them).  Its
+        // blocks come in ascending order, so a key beats the fourth exactly when its value is strictly larger: of equal values
+        // the earlier block stays, which is the reference's rule
+        const u64 none = tk_key(-3.0e38f, 0xffffffffu);
+        u64 best[4] = {none, none, none, none};
         for (u32 i = tid; i < n_ob; i += 256) {
-            float x = row[i];
-            if (x != x) x = -3.0e38f;
-            if (x > lv[3]) {
-                lv[3] = x;
-                li[3] = i;
+            const float x = row[i];
+            const u64 key = tk_key(x != x ? -3.0e38f : x, i);
+            if (key > best[3]) {
+                best[3] = key;
 #pragma unroll
-                for (int k = 3; k > 0; k--)
-                    if (lv[k] > lv[k - 1] || (lv[k] == lv[k - 1] && li[k] < li[k - 1])) {
-                        const float tv = lv[k];
-                        lv[k] = lv[k - 1];
-                        lv[k - 1] = tv;
-                        const u32 ti = li[k];
-                        li[k] = li[k - 1];
-                        li[k - 1] = ti;
-                    }
+                for (int q = 3; q > 0; q--) {
+                    const u64 hi = max(best[q - 1], best[q]), lo = min(best[q - 1], best[q]);
+                    best[q - 1] = hi;
+                    best[q] = lo;
+                }
             }
         }
 #pragma unroll
-        for (int k = 0; k < 4; k++) cand[tid * 4 + k] = tk_key(lv[k], li[k]);
+        for (int q = 0; q < 4; q++) cand[tid * 4 + q] = best[q];
     }
     __syncthreads();
     u64 mine = cand[tid];

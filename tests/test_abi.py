@@ -125,3 +125,18 @@ def test_grid_table_copies_are_identical():
     a = nums(os.path.join(ROOT, "oracle", "iq3s_grid.inc"))
     b = nums(os.path.join(ROOT, "shadow_engine_amd", "kernels", "iq_tables.hip.h"))
     assert len(a) == 512 and a == b
+
+
+def test_the_exl3_heads_lds_bound_is_what_the_kernel_takes():
+    """head_exl3_K: four 4-row rings (static) + 4 KiB of A rows for every 512 inputs and two rows (dynamic), against the 160 KiB of
+    a compute unit: hidden 4096 takes 8 rows at every rate (exactly 160 KiB at K = 8), hidden 8192 at most 4."""
+    L = sz.lib()
+    ring = lambda k: 4 * 4 * 64 * (4 if k in (3, 4) else k) * 4
+    for k in range(1, 9):
+        for hidden in (128, 2048, 2560, 4096, 8192):
+            for m in range(1, 9):
+                want = ring(k) + 4096 * ((hidden // 128 + 3) // 4) * ((m + 1) // 2)
+                assert L.sz_exl3_head_lds_bytes(sz.EXL3(k), hidden, m) == want
+    assert L.sz_exl3_head_lds_bytes(sz.EXL3(8), 4096, 8) == 160 * 1024
+    assert L.sz_exl3_head_lds_bytes(sz.EXL3(4), 8192, 5) > 160 * 1024 >= L.sz_exl3_head_lds_bytes(sz.EXL3(4), 8192, 4)
+    assert L.sz_exl3_head_lds_bytes(sz.Q8_0, 4096, 8) == 0

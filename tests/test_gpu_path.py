@@ -422,10 +422,41 @@ def test_moe_layer_with_masked_experts_matches_the_oracle(gpu, ty):
         assert rel_l2(got[j], want[j]) <= REL_L2, f"row {j}: {rel_l2(got[j], want[j])}"
 
 
-def run_moe_layer_case(gpu, ty, hidden, ff, ne, k, m, shared):
+# What the matrix-core forms of the EXL3 layer are held to (sz_session_set_expert_mode): mode 1 multiplies the codebook's own
+# f16 values and differs from the exact kernels in the order of the f32 additions and in the 22 bits kept of an input; mode 2
+# leaves out every weight's rounding to f16 (half a unit in its last place) and is held to the path's 1e-3.  Measured worst
+# cases over the cases below: mode 1 3.7e-7 relative L2 and 4.6e-7 of the largest output; mode 2 4.3e-4 and 5.2e-4 (the
+# reference holds its own tensor-core EXL3 kernels to 3e-3 of the largest output, crates/shadowzero-cuda/tests/exl3.rs:201).
+MODE_BOUND = {0: REL_L2, 1: 2e-6, 2: REL_L2}
+
+
+@pytest.mark.parametrize("mode", [1, 2])
+@pytest.mark.parametrize("ty,hidden,ff,ne,k,m,shared", [
+    (sz.EXL3(3), 2048, 512, 48, 10, 4, True),
+    (sz.EXL3(2), 2048, 512, 24, 10, 3, True),
+    (sz.EXL3(4), 512, 256, 8, 4, 8, True),         # every expert used by several tokens: items of up to 8 rows
+    (sz.EXL3(3), 256, 256, 6, 6, 2, False),        # k = ne: every expert chosen; no shared expert
+    (sz.EXL3(3), 512, 1024, 12, 4, 3, True),       # ff > 512: the down product's inputs are split, launch 3 sums the partials
+    (sz.EXL3(2), 256, 256, 20, 16, 2, True),       # k = 16
+    (sz.EXL3(4), 3072, 768, 8, 3, 5, True),        # hidden not a multiple of 1024, ff not of 512: workgroups with idle waves; items of 5 rows
+    (sz.EXL3(1), 512, 256, 8, 3, 2, True),         # the other bit rates
+    (sz.EXL3(5), 512, 256, 8, 3, 4, True),
+    (sz.EXL3(6), 256, 512, 6, 2, 3, False),        # K > 5: a tile's windows need two funnel shifts
+    (sz.EXL3(7), 256, 256, 6, 2, 1, True),
+    (sz.EXL3(8), 1024, 256, 6, 3, 4, True),
+    (sz.EXL3(3), 2048, 512, 512, 10, 8, True),     # the benchmark's layer at the most rows a verify batch takes
+    (sz.EXL3(4), 2048, 512, 512, 10, 4, True),     # and at the rows the configurations name
+])
+def test_moe_layer_on_the_matrix_cores(gpu, mode, ty, hidden, ff, ne, k, m, shared):
+    worst = run_moe_layer_case(gpu, ty, hidden, ff, ne, k, m, shared, mode)
+    print(f"mode {mode}: worst relative L2 {worst[0]:.3g}, worst max|dy| / max|y| {worst[1]:.3g}", flush=True)
+
+
+def run_moe_layer_case(gpu, ty, hidden, ff, ne, k, m, shared, mode=0):
     rng = np.random.default_rng(ty * 31 + ne + m)
     dbuf, stride, blobs, sh = build_layer(gpu, rng, ty, hidden, ff, ne, shared)
     s = sz.Session(hidden, ff, ne, k, 1, 0, 8)
+    s.set_expert_mode(mode)
     s.set_layer(0, ty, dbuf.data_ptr(), stride, ty if shared else 0, dbuf.data_ptr() + ne * stride if shared else 0)
     u = rng.normal(size=(m, hidden)).astype(np.float32)
     logits = rng.normal(size=(m, ne)).astype(np.float32)
@@ -440,12 +471,13 @@ def run_moe_layer_case(gpu, ty, hidden, ff, ne, k, m, shared):
     assert np.array_equal(idx, widx), "expert routing must be bit-exact (ids and order)"
     assert np.allclose(w, ww, rtol=2e-6, atol=0)
     for j in range(m):
-        assert rel_l2(got[j], want[j]) <= REL_L2, f"row {j}: {rel_l2(got[j], want[j])}"
+        assert rel_l2(got[j], want[j]) <= MODE_BOUND[mode], f"row {j}: {rel_l2(got[j], want[j])}"
     # twice the same bits (deterministic reductions)
     dy2 = gpu.zeros((m, hidden), dtype=gpu.float32, device="cuda")
     s.moe_layer_verify(0, m, du.data_ptr(), dl.data_ptr(), dg.data_ptr(), dy2.data_ptr())
     gpu.cuda.synchronize()
     assert np.array_equal(bits(dy2.cpu().numpy()), bits(got))
+    return (max(rel_l2(got[j], want[j]) for j in range(m)), max(float(np.abs(got[j] - want[j]).max() / np.abs(want[j]).max()) for j in range(m)))
 
 
 @pytest.mark.parametrize("ty,hidden,ff,ne,k,m", [
@@ -718,7 +750,8 @@ def clear_gap(v, rank=1):
 
 
 @pytest.mark.parametrize("kb,m,hidden,vocab", [(1, 2, 256, 512), (2, 3, 512, 1024), (3, 1, 512, 1024), (3, 8, 512, 1024), (4, 5, 768, 640),
-                                              (5, 4, 512, 1024), (6, 7, 256, 512), (7, 2, 256, 256), (8, 8, 512, 1024), (4, 4, 2560, 1280)])
+                                              (5, 4, 512, 1024), (6, 7, 256, 512), (7, 2, 256, 256), (8, 8, 512, 1024), (4, 4, 2560, 1280),
+                                              (4, 8, 4096, 512), (8, 8, 4096, 256)])   # 144 and 160 KiB of LDS a workgroup: the most a call may take
 def test_exl3_head_argmax_logits_and_top_64_match_the_oracle(gpu, kb, m, hidden, vocab):
     """The lm_head of an EXL3 checkpoint (session.rs:7179-7187): fused arg-max ids bit-exact with the oracle's arg-max, logits
     within the reference's 2e-4 max|y| (tests/exl3.rs:45), the top 64 in the oracle's order; any whole rate, 1..8 rows."""
@@ -803,7 +836,14 @@ def test_exl3_head_full_size(gpu, kb, m):
         assert got_ids[j] == O.argmax(want)
         vals, tids = top[j]
         wv, wi = O.topk(want)
-        assert tids[0] == wi[0] and rel_l2(vals, wv) <= REL_L2 and len(set(tids.tolist()) & set(wi.tolist())) >= 62
+        # the order must be the oracle's as far down as its neighbours are further apart than f32 summation noise; the ids
+        # behind that prefix may swap places with a neighbour, so as a set all but the last few are the oracle's
+        n_clear = 0
+        while n_clear < 64 and clear_gap(want, n_clear + 1):
+            n_clear += 1
+        print(f"row {j}: the first {n_clear} ranks are clear of noise", flush=True)
+        assert n_clear >= 1 and np.array_equal(tids[:n_clear], wi[:n_clear]) and rel_l2(vals, wv) <= REL_L2
+        assert len(set(tids.tolist()) & set(wi.tolist())) >= 62
 
 
 def test_verify_round_with_an_exl3_head(gpu):
@@ -953,14 +993,17 @@ def test_head_top_hands_over_the_sorted_top_64(gpu):
 
 
 # ------------------------------------------------------------------------------------------------- the verify round
-@pytest.mark.parametrize("m", [4, 1, 2, 8])
-def test_verify_round_small_with_planted_drafts(gpu, m):
+@pytest.mark.parametrize("m,mode", [(4, 0), (1, 0), (2, 0), (8, 0), (4, 1), (4, 2), (1, 2), (8, 2), (5, 1)])
+def test_verify_round_small_with_planted_drafts(gpu, m, mode):
     """Three EXL3 layers of mixed bit rates, a Q8_0 head, and the m - 1 drafts planted so that 0, 1, .. and all of them are
-    accepted; the round replayed as a graph gives the bits of the layer-by-layer calls every time."""
+    accepted; the round replayed as a graph gives the bits of the layer-by-layer calls every time (inside a round a layer's
+    rank-order sum rides the next layer's first launch and the layers alternate between two plan buffers; a single call
+    launches it itself).  In every mode of the expert products: the exact kernels (0) and the two matrix-core forms."""
     rng = np.random.default_rng(77 + m)
     hidden, ff, ne, k, vocab = 512, 256, 12, 4, 3000
     rates = [2, 3, 4]
     s = sz.Session(hidden, ff, ne, k, len(rates), vocab, 8)
+    s.set_expert_mode(mode)
     keep_alive, host = [], []
     for l, kb in enumerate(rates):
         dbuf, stride, blobs, sh = build_layer(gpu, rng, sz.EXL3(kb), hidden, ff, ne, True)
@@ -1007,6 +1050,8 @@ def test_verify_round_small_with_planted_drafts(gpu, m):
             assert o[0] == 1 + accepted == O.accept(want_ids[:m - 1], drafts), "accepted-draft count must be bit-exact"
             assert o[1] == want_ids[accepted]
             assert np.array_equal(bits(y.cpu().numpy()), bits(y_ref)), f"replay {replay}"
+    idx, _ = s.last_route(m, stream.handle)                  # the round's last layer, whichever plan buffer it took
+    assert np.array_equal(idx, oracle_layer(sz.EXL3(rates[-1]), hidden, ff, k, host[-1][0], host[-1][1], rl[-1], sgl[-1], u[-1])[1])
 
 
 # ------------------------------------------------------------------------------------------------ run-time compile
@@ -1074,10 +1119,19 @@ def test_the_library_compiles_its_own_kernel_files_at_run_time_in_a_fresh_proces
     t0 = time.time()
     p = subprocess.Popen([sys.executable, "-u", "-c", "import __graft_entry__ as g; g.smoke()"], cwd=root, env=env,
                          stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
-    while p.poll() is None:
-        time.sleep(5)
-        print("run-time compile: %.0f s" % (time.time() - t0), flush=True)
-    out = p.stdout.read()
+    out, limit = "", 900.0
+    while True:
+        # the pipe is drained while the child runs (a child that prints more than a pipe holds would otherwise never end) and
+        # a child that does not end is killed, with what it printed in the failure
+        try:
+            out += p.communicate(timeout=5)[0]
+            break
+        except subprocess.TimeoutExpired as e:
+            print("run-time compile: %.0f s" % (time.time() - t0), flush=True)
+            if time.time() - t0 > limit:
+                p.kill()
+                out += p.communicate()[0] or ""
+                pytest.fail("the child did not end within %.0f s; it printed:\n%s" % (limit, out[-3000:]))
     assert p.returncode == 0 and "smoke ok" in out, out[-3000:]
     import ctypes as C
     lib = sz.lib()
@@ -1157,6 +1211,7 @@ def test_prefill_chunk_matches_the_int8_oracle(gpu, tokens, hidden, ff, ne, k, s
             acc = acc + np.float32(1.0 / (1.0 + np.exp(-np.float64(sgl[j])))) * out
         assert rel_l2(got[j], acc) <= REL_L2, f"token {j}: {rel_l2(got[j], acc)}"
     # H codes: the same rounding rule on values that agree to the last bit or two of f32 (device expf against libm's, fused fold)
+    print(f"H codes: {code_diff} of {code_total} differ from the oracle's ({code_diff / code_total:.2e} of the places)", flush=True)
     assert code_diff <= 1e-3 * code_total, f"{code_diff} of {code_total} H codes differ"
 
 
@@ -1202,8 +1257,14 @@ def test_config4_prefill_chunk_full_size(gpu):
     sz.check(sz.lib().sz_download(xq.ctypes.data, s.prefill_buffer(0), xq.nbytes))
     wq_all, wd_all, _ = O.quantize_act(x, 32)
     assert np.array_equal(xq.ravel(), wq_all)
+    wts = np.empty((tokens, k), np.float32)
+    sz.check(sz.lib().sz_download(wts.ctypes.data, s.prefill_buffer(3), wts.nbytes))
     for j in range(tokens):
-        assert np.array_equal(tidx[j], O.route(logits[j], k)[0]), f"token {j}"
+        oi, ow = O.route(logits[j], k)
+        assert np.array_equal(tidx[j], oi), f"token {j}"
+        # the chunk's weights are ex_t over the sum of the chosen ex (the reference divides every ex by the sum over all experts
+        # first, forward.rs:1143-1147): the same value before rounding, within a unit in the last place of f32 after it
+        assert np.allclose(wts[j], ow, rtol=2e-6, atol=0), f"token {j}"
     counts = np.bincount(tidx.ravel(), minlength=ne)
     print("distinct experts hit:", int((counts > 0).sum()), "largest group:", int(counts.max()), flush=True)
     assert counts.max() > 64, "the skew must give an expert more than one pass of 64 tokens"
@@ -1261,8 +1322,8 @@ def test_prefill_chunk_of_the_largest_size_equals_its_parts(gpu):
 
 def test_config5_full_depth_verify_round(gpu):
     """48 layers of 512 + 1 EXL3 experts at mixed rates (about 29 GB generated in HBM), a 4-token batch, the 151,936-row Q8_0
-    head, arg-max and acceptance: token ids and the accepted count exact against the oracle, every layer's output of one
-    token (all four for the first layer of each rate) within 1e-3."""
+    head, arg-max and acceptance: token ids and the accepted count exact against the oracle, every layer's output of two
+    tokens (all four for the first layer of each rate) within 1e-3."""
     from shadow_engine_amd import synth_device
     torch = gpu
     free, _total = torch.cuda.mem_get_info()
@@ -1307,7 +1368,7 @@ def test_config5_full_depth_verify_round(gpu):
         oty = O.exl3_type(kb)
         shape = O.expert_shape(oty, oty, hidden, ff)
         nb = shape.gate_bytes + shape.up_bytes + shape.down_bytes
-        toks = range(m) if kb not in seen_rates else [l % m]
+        toks = range(m) if kb not in seen_rates else [l % m, (l + 1) % m]
         seen_rates.add(kb)
         for j in toks:
             ids = synth_device.route_ids(rl_h[l, j:j + 1], k)[0]
