@@ -232,6 +232,40 @@ def iq3s_prefill(torch, sz, synth, synth_device, stream, tokens=512):
     return w
 
 
+def exl3_prefill(torch, sz, synth, synth_device, stream, tokens=512, bits=3):
+    """The prefill chunk of config 4 through the verify round's kind of experts: EXL3 at `bits` bits a weight, f16 activations on the
+    rows of the matrix instruction (no int8 quantization), the shared expert included."""
+    w = Workload()
+    sess = sz.Session(HIDDEN, FF, NE, TOPK, 1, 0, 8)
+    buf, stride = synth_device.exl3_layer(torch, 4400, HIDDEN, FF, NE, bits)
+    sess.set_layer(0, sz.EXL3(bits), buf.data_ptr(), stride, sz.EXL3(bits), buf.data_ptr() + NE * stride)
+    rng = np.random.default_rng(4)
+    logits = synth.zipf_router_logits(rng, tokens, NE)
+    g = torch.Generator(device="cuda")
+    g.manual_seed(13)
+    x = torch.randn((tokens, HIDDEN), device="cuda", generator=g)
+    rl = torch.from_numpy(logits).cuda()
+    sgl = torch.randn(tokens, device="cuda", generator=g)
+    y = torch.zeros((tokens, HIDDEN), device="cuda")
+    w.step = lambda: sess.moe_prefill_chunk(0, tokens, x.data_ptr(), rl.data_ptr(), sgl.data_ptr(), y.data_ptr(), stream.handle)
+    ids = synth_device.route_ids(logits, TOPK)
+    distinct = int(np.unique(ids).size) + 1
+    pairs = tokens * (TOPK + 1)
+    zs = HIDDEN // 512
+    gu, dn = 2 * synth.exl3_blob_len(HIDDEN, FF, bits), synth.exl3_blob_len(FF, HIDDEN, bits)
+    w.step_bytes = distinct * (gu + dn) + tokens * (2 * HIDDEN + NE) * 4
+    w.kernel_bytes = {"prefill_gate_up_exl3_%d" % bits: distinct * gu + tokens * HIDDEN * 4 + pairs * 2 * zs * FF * 4,
+                      "prefill_down_exl3_%d" % bits: distinct * dn + pairs * 2 * zs * FF * 4 + pairs * HIDDEN * 4}
+    w.dtype = "f32 accumulate over EXL3 f16 codebook weights x f16 activations (matrix cores)"
+    w.describe = {"workload": "prefill chunk, %d tokens x hidden 2048 through 512 EXL3 K=%d experts + the shared one (top-10, Zipf-skewed routing, "
+                              "%d distinct experts hit), f16 activations" % (tokens, bits, distinct), "rows": tokens, "resident_GB": round(buf.numel() / 1e9, 2)}
+    w.counters_key = "exl3prefill" if (tokens == 512 and bits == 3) else None
+    rl_h = logits[:1]
+    w.cpu = ("exl3_token", ((buf, stride), bits, rl_h, x[:1].cpu().numpy(), sgl[:1].cpu().numpy()))
+    w.keep = (sess, buf, x, rl, sgl, y)
+    return w
+
+
 def exl3_head(torch, sz, synth, synth_device, stream, bits):
     """The lm_head of an EXL3 checkpoint: 151936 x 2048 at `bits` bits a weight for a verify batch, arg-max fused in."""
     w = Workload()
@@ -578,10 +612,12 @@ def build_workload(name, torch, sz, synth, synth_device, stream, args):
         return iq3s_decode(torch, sz, synth, synth_device, stream)
     if name == "config4":
         return iq3s_prefill(torch, sz, synth, synth_device, stream, args.tokens)
+    if name == "exl3prefill":
+        return exl3_prefill(torch, sz, synth, synth_device, stream, args.tokens, args.bits or 3)
     if name == "exl3head":
-        return exl3_head(torch, sz, synth, synth_device, stream, args.bits)
+        return exl3_head(torch, sz, synth, synth_device, stream, args.bits or 4)
     if name == "exl3top":
-        return exl3_head_top(torch, sz, synth, synth_device, stream, args.bits, args.screen)
+        return exl3_head_top(torch, sz, synth, synth_device, stream, args.bits or 4, args.screen)
     if name == "stage":
         return stage_exl3_layer(torch, sz, synth, stream)
     return snapshot_states(torch, sz, stream)
@@ -593,10 +629,10 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--layers", type=int, default=48)
-    ap.add_argument("--workload", default="config5", choices=["config1", "config2", "config3", "config4", "config5", "exl3head", "exl3top", "stage", "snapshot"])
+    ap.add_argument("--workload", default="config5", choices=["config1", "config2", "config3", "config4", "config5", "exl3prefill", "exl3head", "exl3top", "stage", "snapshot"])
     ap.add_argument("--rows", type=int, default=4, help="rows of the verify batch (config3, config5, exl3head; the configurations name 4; 1..8)")
     ap.add_argument("--tokens", type=int, default=512, help="tokens of the prefill chunk (config4 only; the configuration names 512)")
-    ap.add_argument("--bits", type=int, default=4, help="bits a weight of the EXL3 head (exl3head, exl3top)")
+    ap.add_argument("--bits", type=int, default=0, help="bits a weight of the EXL3 head (exl3head, exl3top: 4 unless given) or of the chunk's experts (exl3prefill: 3)")
     ap.add_argument("--screen", type=int, default=0, help="exl3top: blocks a row of the inexact 2-bit screen (0: the exact hand-off)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true", help="default workload only: do not time configurations 1-4 after it")

@@ -328,7 +328,7 @@ struct sz_session {
         DevBuf w_q2, w_sc, xq, x_sc, x_corr, bmax, seen, sel, logits;
     } hp;
     struct {
-        DevBuf xq, xd, tidx, w, cnt, offs, list, items, hq, hd, eo;
+        DevBuf xq, xd, tidx, w, cnt, offs, list, items, hq, hd, eo, gup;
     } pf;   // the prefill chunk's buffers, grown on demand
     void* top_host = nullptr;  // pinned host memory the top-64 merge writes to directly (8 rows of 128 words): no copy back
     bool last_fused = false;   // the last layer call left its routing in the fused layout [tidx | w | cnt]
@@ -1069,12 +1069,51 @@ int32_t sz_moe_prefill_chunk(sz_session* s, uint32_t l, uint32_t tokens, uint64_
     const sz_session_config& c = s->cfg;
     if (l >= s->layers.size() || !s->layers[l].set) return fail("sz_moe_prefill_chunk: layer " + std::to_string(l) + " has no experts set");
     SzLayer& L = s->layers[l];
-    if (L.type != SZ_TYPE_IQ3_S || (L.shared && L.shared_type != SZ_TYPE_IQ3_S)) return fail("sz_moe_prefill_chunk: the int8 MFMA path is built for IQ3_S experts");
+    Format f;
+    std::string tag;
+    format_of(L.type, f, tag);
+    const bool exl3 = f.exl3 && !f.half;
+    if ((L.type != SZ_TYPE_IQ3_S && !exl3) || (L.shared && L.shared_type != L.type))
+        return fail("sz_moe_prefill_chunk: the chunk kernels are built for IQ3_S experts (int8 activations) and EXL3 experts at a whole bit rate");
     if (tokens == 0 || tokens > 16384) return fail("sz_moe_prefill_chunk: " + std::to_string(tokens) + " tokens (1..16384)");   // BIG_BATCH_MAX, session.rs:191
     if (c.hidden % 256 || c.ff % 256 || (x & 15) || (y & 15)) return fail("sz_moe_prefill_chunk: shapes must be multiples of 256 and 16-byte aligned");
     const bool shared = L.shared != 0;
     const uint64_t T = tokens, k = c.top_k, np = T * k, rows = np + (shared ? T : 0);
     auto& pb = s->pf;
+    if (exl3) {
+        // EXL3 experts: f16 activations on the rows of the matrix instruction, both rotations on the matrix cores, items of up to
+        // 32 pairs (kernels/exl3.hip, "the prefill chunk of an EXL3 layer")
+        if (c.ff > 512) return fail("sz_moe_prefill_chunk: EXL3 experts of more than 512 intermediate features are not built (the down launch keeps four 128-blocks of a token)");
+        const uint32_t zs = (c.hidden / 128 + 3) / 4;
+        const uint64_t max_items = c.n_expert + 1 + rows / 32;
+        if (pb.tidx.need(np * 4) || pb.w.need(np * 4) || pb.cnt.need(T * 4) || pb.offs.need((c.n_expert + 2) * 4ull) || pb.list.need(rows * 4) ||
+            pb.items.need((2 + 4 * max_items) * 4) || pb.gup.need(2ull * rows * zs * c.ff * 4) || pb.eo.need(rows * c.hidden * 4))
+            return 1;
+        const uint64_t sh = shared ? L.eaddr.ptr + 3ull * c.n_expert * 8 : 0, items_d = pb.items.ptr + (1 + 2 * max_items) * 4;
+        {
+            const sz_arg a[] = {P(rl), P(pb.tidx.ptr), P(pb.w.ptr), U32(c.n_expert), U32(c.top_k), U32(tokens)};
+            if (launch("route_topk_rows", (tokens + 3) / 4, 1, 1, 256, 0, stream, a)) return 1;
+        }
+        {
+            const sz_arg a[] = {P(pb.tidx.ptr), U32(tokens), U32(c.top_k), U32(c.n_expert), U32(shared ? tokens : 0), P(pb.offs.ptr), P(pb.list.ptr), P(pb.cnt.ptr),
+                                P(pb.items.ptr), P(items_d), U32(32), U32(32)};
+            if (launch("prefill_group", 1, 1, 1, 1024, 0, stream, a)) return 1;
+        }
+        const uint32_t stride = (f.bits == 3 || f.bits == 4) ? 4 : (uint32_t) f.bits;
+        const uint32_t lds = 4 * (4 * 8 * 32 * 8 + 4 * (4 * 64 * stride) + 2 * 32 + 4 * 32 + 4 * 16);   // XPF_LDS_WORDS
+        {
+            const sz_arg a[] = {P(L.eaddr.ptr), P(sh), P(pb.offs.ptr), P(pb.list.ptr), P(pb.items.ptr), P(x), P(pb.gup.ptr), U32(c.n_expert), U32(c.top_k),
+                                U32((uint32_t) np), U32((uint32_t) rows), U32(c.hidden), U32(c.ff)};
+            if (launch(("prefill_gate_up_" + tag).c_str(), (uint32_t) max_items, 2 * zs, 1, 256, lds, stream, a)) return 1;
+        }
+        {
+            const sz_arg a[] = {P(L.eaddr.ptr), P(sh), P(pb.offs.ptr), P(pb.list.ptr), P(items_d), P(pb.gup.ptr), P(pb.eo.ptr), U32(c.n_expert), U32(c.top_k),
+                                U32((uint32_t) np), U32((uint32_t) rows), U32(c.hidden), U32(c.ff), U32(zs)};
+            if (launch(("prefill_down_" + tag).c_str(), (uint32_t) max_items, (c.hidden / 128 + 3) / 4, 1, 256, lds, stream, a)) return 1;
+        }
+        const sz_arg a[] = {P(y), P(pb.eo.ptr), P(pb.w.ptr), P(shared ? pb.eo.ptr + np * c.hidden * 4 : 0), P(sgl), P(pb.cnt.ptr), U32(c.hidden), U32(c.top_k)};
+        return launch("moe_combine_qwen_rows", (c.hidden + 255) / 256, tokens, 1, 256, 0, stream, a);
+    }
     const uint64_t max_items = c.n_expert + 1 + rows / 64, max_items_d = c.n_expert + 1 + rows / 32;   // every expert's runs of up to 64 (32) pairs: PF_TOK, PF_TOK_D in kernels/prefill.hip
     if (pb.xq.need(T * c.hidden) || pb.xd.need(T * c.hidden / 32 * 4) || pb.tidx.need(np * 4) || pb.w.need(np * 4) || pb.cnt.need(T * 4) ||
         pb.offs.need((c.n_expert + 2) * 4ull) || pb.list.need(rows * 4) || pb.items.need((2 + 2 * max_items + 2 * max_items_d) * 4) || pb.hq.need(rows * c.ff) || pb.hd.need(rows * (c.ff / 32) * 4) ||
@@ -1089,7 +1128,7 @@ int32_t sz_moe_prefill_chunk(sz_session* s, uint32_t l, uint32_t tokens, uint64_
     }
     const uint64_t items_d = pb.items.ptr + (1 + 2 * max_items) * 4;   // the down kernel's items: runs of up to 32 pairs (PF_TOK_D)
     {
-        const sz_arg a[] = {P(pb.tidx.ptr), U32(tokens), U32(c.top_k), U32(c.n_expert), U32(shared ? tokens : 0), P(pb.offs.ptr), P(pb.list.ptr), P(pb.cnt.ptr), P(pb.items.ptr), P(items_d)};
+        const sz_arg a[] = {P(pb.tidx.ptr), U32(tokens), U32(c.top_k), U32(c.n_expert), U32(shared ? tokens : 0), P(pb.offs.ptr), P(pb.list.ptr), P(pb.cnt.ptr), P(pb.items.ptr), P(items_d), U32(64), U32(32)};
         if (launch("prefill_group", 1, 1, 1, 1024, 0, stream, a)) return 1;
     }
     {

@@ -1769,3 +1769,465 @@ EXL3_LINW_ENTRIES(5)
 EXL3_LINW_ENTRIES(6)
 EXL3_LINW_ENTRIES(7)
 EXL3_LINW_ENTRIES(8)
+
+// ------------------------------------------------------------------------ the prefill chunk of an EXL3 layer (matrix cores)
+// A chunk's tokens grouped by expert (prefill_group in kernels/prefill.hip: runs of up to 32 (token, rank) pairs of one
+// expert are a work item) through gate/up and down with the item's tokens on the rows of the matrix instruction: an
+// expert's weights are decoded once for up to 32 tokens (the reference's mma_grouped_exl3_pre_K, kernels/exl3.cu:684,704,724,
+// with groups of 64, session.rs:5159-5189).  Both rotations of the format run on the matrix cores too: (x * suh) H is a
+// product with the 128 x 128 matrix of signs, whose 16 x 16 x 16 operands a lane makes from its own lane number (H[i][j] =
+// (-1)^popcount(i & j): a tile of it is a per-lane pattern times the parity of the two tile numbers), so a token's rotation
+// costs 4 matrix instructions a 128-block instead of the 130 vector instructions of the butterflies.  Inputs ride as single
+// f16 values scaled by a power of two per token and workgroup (the reference converts to f16 unscaled); weights are the
+// codebook's own f16 values; sums are f32.  Against the exact arithmetic the f16 roundings of the activations cost about
+// 3e-4 relative L2 of a layer's output (bound of the path: 1e-3).
+
+#define XPF_TOK 32
+
+// The lane's share of a sign tile of H for the rotation product: element q of the pair is H[16 ks + 4 a + q][16 ct + n] for
+// tile numbers of even popcount(ks & ct) (a = lane / 16, n = lane % 16); the other tiles are the negative.
+__device__ __forceinline__ void xpf_sign_tile(u32 lane, u32 (&hop)[2]) {
+    const u32 n = lane & 15, a = lane >> 4;
+    u32 h[4];
+#pragma unroll
+    for (u32 q = 0; q < 4; q++) h[q] = (__builtin_popcount((4 * a + q) & n) & 1) ? 0xbc00u : 0x3c00u;   // -1.0 : +1.0
+    hop[0] = h[0] | (h[1] << 16);
+    hop[1] = h[2] | (h[3] << 16);
+}
+
+// rot[ct][q] = sum over the 128 inputs i of v[token][i] H[i][16 ct + n] for token 4 a + q of the tile: v comes as load4(ks) =
+// the lane's token's (lane % 16) inputs 16 ks + 4 a .. + 3 (already times the input scales), rounded to f16 here.
+template <class F>
+__device__ __forceinline__ void xpf_rotate_tile(F&& load4, const u32 (&hop)[2], f32x4 (&rot)[8]) {
+#pragma unroll
+    for (int ct = 0; ct < 8; ct++) rot[ct] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+    const u32x2 hp = {hop[0], hop[1]}, hn = {hop[0] ^ 0x80008000u, hop[1] ^ 0x80008000u};
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++) {
+        const f32x4 v = load4(ks);
+        const f16x4 av = {(_Float16) v[0], (_Float16) v[1], (_Float16) v[2], (_Float16) v[3]};
+#pragma unroll
+        for (int ct = 0; ct < 8; ct++) {
+            const bool neg = __builtin_popcount(ks & ct) & 1;
+            rot[ct] = __builtin_amdgcn_mfma_f32_16x16x16f16(av, __builtin_bit_cast(f16x4, neg ? hn : hp), rot[ct], 0, 0, 0);
+        }
+    }
+}
+
+// The power of two that takes the largest magnitude of the lane's token's (lane % 16) 128 inputs to [2^14, 2^15), so that they
+// round to f16 without overflow or loss of small values, and its inverse: v = the lane's 32 of them (the other 96 are in
+// lanes + 16, + 32, + 48).
+__device__ __forceinline__ void xpf_input_scale(const f32x4 (&v)[8], u32 lane, float& scale, float& inv) {
+    float m = 0.0f;
+#pragma unroll
+    for (int ks = 0; ks < 8; ks++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) m = fmaxf(m, __builtin_fabsf(v[ks][q]));
+    m = fmaxf(m, lane_xor<16>(m, lane));
+    m = fmaxf(m, lane_xor<32>(m, lane));
+    pow2_scale_of(f32_bits(m), scale, inv);
+}
+
+// The largest magnitude of each of the lane's four tokens (4 a + q) over the tile's 128 rotated values: over the lane's 8
+// column tiles, then over the 16 lanes of its row.
+__device__ __forceinline__ void xpf_token_max(const f32x4 (&rot)[8], float (&mx)[4]) {
+#pragma unroll
+    for (int q = 0; q < 4; q++) {
+        float m = 0.0f;
+#pragma unroll
+        for (int ct = 0; ct < 8; ct++) m = fmaxf(m, __builtin_fabsf(rot[ct][q]));
+        m = fmaxf(m, bits_f32(__builtin_amdgcn_update_dpp(0u, f32_bits(m), 0xb1, 0xf, 0xf, true)));    // quad_perm [1,0,3,2]
+        m = fmaxf(m, bits_f32(__builtin_amdgcn_update_dpp(0u, f32_bits(m), 0x4e, 0xf, 0xf, true)));    // quad_perm [2,3,0,1]
+        m = fmaxf(m, bits_f32(__builtin_amdgcn_update_dpp(0u, f32_bits(m), 0x124, 0xf, 0xf, true)));   // row_ror:4
+        m = fmaxf(m, bits_f32(__builtin_amdgcn_update_dpp(0u, f32_bits(m), 0x128, 0xf, 0xf, true)));   // row_ror:8
+        mx[q] = m;
+    }
+}
+
+// A tile's rotation with its inputs brought into f16's range first: every token's inputs times its own power of two, the
+// transform, and the rotated values times the inverse (exact both ways).  pre: 16 floats of the wave's own LDS.
+__device__ __forceinline__ void xpf_rotate_scaled(f32x4 (&v)[8], const u32 (&hop)[2], f32x4 (&rot)[8], float* pre, u32 lane) {
+    float scale, inv;
+    xpf_input_scale(v, lane, scale, inv);
+    if (lane < 16) pre[lane] = inv;
+    xpf_rotate_tile([&](int ks) { return v[ks] * scale; }, hop, rot);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+    const f32x4 iv = *(const f32x4*) (pre + 4 * (lane >> 4));   // of the lane's tokens 4 a + q
+#pragma unroll
+    for (int ct = 0; ct < 8; ct++) rot[ct] *= iv;
+    __builtin_amdgcn_wave_barrier();                             // the strip is free for the next tile
+}
+
+// The tile's rotated values as A rows of the products: f16(rot * sc[q]) at arows[(ct * XPF_TOK + 16 T + 4 a + q) * 16 + slot of n]
+// (tile row ct of the 128-block, A row = the token's place in the item).
+__device__ __forceinline__ void xpf_put_a_rows(u16* arows, u32 T, const f32x4 (&rot)[8], const float (&sc)[4], u32 lane) {
+    const u32 n = lane & 15, a = lane >> 4;
+    u16* at = arows + (16 * T + 4 * a) * 16 + exl3_aslot(n);
+#pragma unroll
+    for (int ct = 0; ct < 8; ct++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) at[(ct * XPF_TOK + q) * 16] = __builtin_bit_cast(u16, (_Float16) (rot[ct][q] * sc[q]));
+}
+
+// The products of one wave: `nrows` tile rows of its 128-column block (the stream starts at row0, its first rows requested
+// by exl3_mma_rows_start) against the A rows at xa (tile row i at xa + i * XPF_TOK * 16, A row = token) for one or two
+// token tiles; acc[T][c] as exl3_wave_mma's (row 4 a + q = token 16 T + 4 a + q).
+template <int K>
+__device__ __forceinline__ void xpf_wave_products(const u32* __restrict__ row0, u64 pitch, u32 nrows, const u32* wb, u32 lds, const u16* xa, bool two,
+                                                  u32 lane, f32x4 (&acc)[2][8]) {
+    constexpr int D = 4;
+    typedef Exl3Rows<K, D> R;
+    constexpr int stride = R::stride, ur = R::unit_rows;
+    constexpr bool one_shift = 16 + 3 * K <= 32;
+    const u32 n16 = lane & 15, a = lane >> 4;
+    const u32 t0 = 32 * (n16 & 7) + 8 * a + 4 * (n16 >> 3);
+    auto window = [&](u32 e, u32& om, u32& op, u32& sh) {
+        const u32 jp = (e - 1) >> 5, jm = (jp + 8 * K - 1) % (8 * K);
+        sh = 31 - ((e - 1) & 31);
+        om = (jm / K) * stride + jm % K;
+        op = (jp / K) * stride + jp % K;
+    };
+    u32 om1, op1, sh1, om0 = 0, op0 = 0, sh0 = 0;
+    window((t0 + 4) * K, om1, op1, sh1);
+    if constexpr (!one_shift) window((t0 + 2) * K, om0, op0, sh0);
+#pragma unroll
+    for (int T = 0; T < 2; T++)
+#pragma unroll
+        for (int c = 0; c < 8; c++) acc[T][c] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    const u16* xa0 = xa + n16 * 16 + 4 * a;
+#pragma unroll 1
+    for (u32 i = 0; i < nrows; i++) {
+        exl3_rows_wait<K, D>(i + D > nrows ? i + D - nrows : 0);
+        const u32* row = wb + (i & (D - 1)) * R::row_words;
+        u32 w1[8][2], w0[8][2];
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            w1[c][0] = row[c * 8 * stride + om1];
+            w1[c][1] = row[c * 8 * stride + op1];
+            if constexpr (!one_shift) {
+                w0[c][0] = row[c * 8 * stride + om0];
+                w0[c][1] = row[c * 8 * stride + op0];
+            }
+        }
+        typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+        const u32x2 xv0 = *(const u32x2*) (xa0 + i * (XPF_TOK * 16));
+        u32x2 xv1 = *(const u32x2*) (xa0 + i * (XPF_TOK * 16) + 16 * 16);
+        if (!two) xv1 = u32x2{0u, 0u};
+        if ((i + 1) % ur == 0 && i + D + 1 - ur < nrows) {
+            __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): the row's words are in registers, its slot can take the row D further on
+            exl3_unit_issue<K, D>(row0, pitch, i + D + 1 - ur, lane, lds);
+        }
+        const f16x4 av0 = __builtin_bit_cast(f16x4, xv0), av1 = __builtin_bit_cast(f16x4, xv1);
+#pragma unroll
+        for (int c = 0; c < 8; c++) {
+            const u32 hi = __builtin_amdgcn_alignbit(w1[c][0], w1[c][1], sh1);
+            u32 s0, s1;
+            if constexpr (one_shift) {
+                s0 = __builtin_amdgcn_ubfe(hi, 3 * K, 16);
+                s1 = __builtin_amdgcn_ubfe(hi, 2 * K, 16);
+            } else {
+                const u32 lo = __builtin_amdgcn_alignbit(w0[c][0], w0[c][1], sh0);
+                s0 = __builtin_amdgcn_ubfe(lo, K, 16);
+                s1 = lo & 0xffffu;
+            }
+            const u32 s2 = __builtin_amdgcn_ubfe(hi, K, 16), s3 = hi & 0xffffu;
+            const f16x2 b01 = exl3_cb2_pair(s0, s1), b23 = exl3_cb2_pair(s2, s3);
+            const f16x4 bv = {b01[0], b01[1], b23[0], b23[1]};
+            acc[0][c] = __builtin_amdgcn_mfma_f32_16x16x16f16(av0, bv, acc[0][c], 0, 0, 0);
+            if (two) acc[1][c] = __builtin_amdgcn_mfma_f32_16x16x16f16(av1, bv, acc[1][c], 0, 0, 0);
+        }
+    }
+}
+
+// The output side of a wave's block: out[c][q] (column 16 c + n of the lane's four tokens 4 a + q of one tile) through the
+// 128-point transform over the columns (three stages over c in registers, four over the lanes of the row of 16) times the
+// output scales sv[c] (column 16 c + n), the 1/sqrt(128) included.
+__device__ __forceinline__ void xpf_output_side(f32x4 (&v)[8], const float (&sv)[8], u32 lane) {
+#pragma unroll
+    for (int h = 1; h < 8; h <<= 1)
+#pragma unroll
+        for (int c = 0; c < 8; c++)
+            if (!(c & h)) {
+                const f32x4 s = v[c] + v[c + h], d = v[c] - v[c + h];
+                v[c] = s;
+                v[c + h] = d;
+            }
+#pragma unroll
+    for (int c = 0; c < 8; c++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            float x = v[c][q];
+            { const float p = lane_xor<1>(x, lane); x = __builtin_fmaf(x, bits_f32(0x3f800000u | ((lane & 1) ? 0x80000000u : 0u)), p); }
+            { const float p = lane_xor<2>(x, lane); x = __builtin_fmaf(x, bits_f32(0x3f800000u | ((lane & 2) ? 0x80000000u : 0u)), p); }
+            { const float p = lane_xor<4>(x, lane); x = __builtin_fmaf(x, bits_f32(0x3f800000u | ((lane & 4) ? 0x80000000u : 0u)), p); }
+            { const float p = lane_xor<8>(x, lane); x = __builtin_fmaf(x, bits_f32(0x3f800000u | ((lane & 8) ? 0x80000000u : 0u)), p); }
+            v[c][q] = x * sv[c];
+        }
+}
+
+// Shared set-up of the two launches: the item, its pairs and rows.  Returns the number of the item's pairs (0: no such item).
+__device__ __forceinline__ u32 xpf_item(const u32* __restrict__ offs, const u32* __restrict__ list, const u32* __restrict__ items, u32 item, u32 ne, bool has_shared,
+                                        u32 k, u32 npairs, u32* s_pairs, u32* s_rows, u32& e) {
+    if (item >= items[0]) return 0;
+    e = items[1 + 2 * item];
+    const u32 t0 = items[2 + 2 * item];
+    if (e == ne && !has_shared) return 0;
+    const u32 first = offs[e], nt = min((u32) XPF_TOK, offs[e + 1] - first - t0);
+    if (threadIdx.x < XPF_TOK) {
+        const u32 p = list[first + t0 + min(threadIdx.x, nt - 1)];   // a place past the item's end repeats its last pair: loads stay in bounds, results are dropped
+        s_pairs[threadIdx.x] = p;
+        s_rows[threadIdx.x] = p < npairs ? p / k : p - npairs;
+    }
+    return nt;
+}
+
+// LDS of a workgroup of the two launches, in words: the A rows of four 128-blocks (32 tokens each), the four waves' rings,
+// the item's pairs and rows, the waves' token maxima, the waves' strips of 16 input scales.
+#define XPF_LDS_WORDS(ring) (4 * 8 * XPF_TOK * 8 + 4 * (ring) + 2 * XPF_TOK + 4 * XPF_TOK + 4 * 16)
+
+// Launch 1: item blockIdx.x, sel = blockIdx.y / zs (gate, up), z = blockIdx.y % zs: the inputs' 128-blocks 4 z .. 4 z + 3.
+// Wave w rotates block 4 z + w of the item's tokens, then takes the 128-column blocks w, w + 4, .. of ff over the four input
+// blocks; partial sums gup[((sel * NP + pair) * zs + z)][ff], already through the output-side transform and scales (NP =
+// npairs + the shared expert's rows).  grid = (bound on the items, 2 zs), block 256, dynamic LDS 4 XPF_LDS_WORDS.
+template <int K>
+__device__ __forceinline__ void prefill_gate_up_exl3_kernel(const u64* __restrict__ eaddr, const u64* __restrict__ sh_addr, const u32* __restrict__ offs,
+                                                            const u32* __restrict__ list, const u32* __restrict__ items, const float* __restrict__ x,
+                                                            float* __restrict__ gup, u32 ne, u32 k, u32 npairs, u32 NP, u32 hidden, u32 ff) {
+    typedef Exl3Rows<K, 4> R;
+    extern __shared__ __attribute__((aligned(16))) u32 dyn[];
+    u16* arows = (u16*) dyn;                                  // [block of the four][tile row][token][16]
+    u32* rings = dyn + 4 * 8 * XPF_TOK * 8;
+    u32* s_pairs = rings + 4 * R::words;
+    u32* s_rows = s_pairs + XPF_TOK;
+    float* s_max = (float*) (s_rows + XPF_TOK);               // [wave][token]
+    float* s_pre = s_max + 4 * XPF_TOK;                       // [wave][16]
+    const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const u32 kbs = hidden / 128, zs = (kbs + 3) / 4, sel = blockIdx.y / zs, z = blockIdx.y - sel * zs;
+    u32 e;
+    const u32 nt = xpf_item(offs, list, items, blockIdx.x, ne, sh_addr != nullptr, k, npairs, s_pairs, s_rows, e);
+    if (nt == 0) return;
+    const bool two = nt > 16;
+    const u8* bp = (const u8*) (e < ne ? eaddr[(u64) sel * ne + e] : sh_addr[sel]);
+    const u32 kb = 4 * z + wave, nkb = min(4u, kbs - 4 * z);
+    __syncthreads();                                          // the item's pairs and rows are written
+    u32 hop[2];
+    xpf_sign_tile(lane, hop);
+    f32x4 rot[2][8];
+    float mx[2][4];
+    if (wave < nkb) {
+        const u16* suh = (const u16*) bp + kb * 128 + 4 * (lane >> 4);
+        typedef u16 u16x4 __attribute__((ext_vector_type(4)));
+        float sc[8][4];
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+            const u16x4 s4 = *(const u16x4*) (suh + 16 * ks);
+#pragma unroll
+            for (int q = 0; q < 4; q++) sc[ks][q] = f16_to_f32(s4[q]);
+        }
+#pragma unroll
+        for (int T = 0; T < 2; T++) {
+            if (T == 1 && !two) break;
+            const float* xr = x + (u64) s_rows[16 * T + (lane & 15)] * hidden + kb * 128 + 4 * (lane >> 4);
+            f32x4 xv[8];
+#pragma unroll
+            for (int ks = 0; ks < 8; ks++) {
+                xv[ks] = *(const f32x4*) (xr + 16 * ks);
+#pragma unroll
+                for (int q = 0; q < 4; q++) xv[ks][q] *= sc[ks][q];
+            }
+            xpf_rotate_scaled(xv, hop, rot[T], s_pre + wave * 16, lane);
+            xpf_token_max(rot[T], mx[T]);
+            if ((lane & 15) == 0) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) s_max[wave * XPF_TOK + 16 * T + 4 * (lane >> 4) + q] = mx[T][q];
+            }
+        }
+    }
+    __syncthreads();
+    // one power of two a token for the workgroup's four blocks; the lane's tokens 16 T + 4 a + q
+    float inv[2][4];
+#pragma unroll
+    for (int T = 0; T < 2; T++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const u32 t = 16 * T + 4 * (lane >> 4) + q;
+            float m = 0.0f;
+            for (u32 w = 0; w < nkb; w++) m = fmaxf(m, s_max[w * XPF_TOK + t]);
+            float scale, iv;
+            pow2_scale_of(f32_bits(m), scale, iv);
+            inv[T][q] = iv;
+            mx[T][q] = scale * 0.08838835f;                   // the factor of the stored values: the power of two and the transform's 1/sqrt(128)
+        }
+    if (wave < nkb) {
+        xpf_put_a_rows(arows + wave * (8 * XPF_TOK * 16), 0, rot[0], mx[0], lane);
+        if (two) xpf_put_a_rows(arows + wave * (8 * XPF_TOK * 16), 1, rot[1], mx[1], lane);
+    }
+    __syncthreads();
+    const u32 wb_lds = __builtin_amdgcn_readfirstlane(lds_offset(rings + wave * R::words));
+    const u64 pitch = (u64) (ff / 16) * EXL3_TILE_WORDS(K, false);
+    for (u32 cb = wave; cb < ff / 128; cb += 4) {
+        const u32* row0 = (const u32*) (bp + 2 * (u64) hidden + 2 * (u64) ff + 4) + ((u64) (4 * z) * 8 * (ff / 16) + cb * 8) * EXL3_TILE_WORDS(K, false);
+        exl3_rows_issue<K, 4>(row0, pitch, lane, wb_lds);     // a stream has at least 8 rows
+        f32x4 acc[2][8];
+        xpf_wave_products<K>(row0, pitch, 8 * nkb, rings + wave * R::words, wb_lds, arows, two, lane, acc);
+        const u16* svh = (const u16*) (bp + 2 * (u64) hidden) + cb * 128 + (lane & 15);
+        float sv[8];
+#pragma unroll
+        for (int c = 0; c < 8; c++) sv[c] = f16_to_f32(svh[16 * c]) * 0.08838835f;
+#pragma unroll
+        for (int T = 0; T < 2; T++) {
+            if (T == 1 && !two) break;
+#pragma unroll
+            for (int c = 0; c < 8; c++)
+#pragma unroll
+                for (int q = 0; q < 4; q++) acc[T][c][q] *= inv[T][q];
+            xpf_output_side(acc[T], sv, lane);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const u32 t = 16 * T + 4 * (lane >> 4) + q;
+                if (t < nt) {
+                    float* o = gup + (((u64) sel * NP + s_pairs[t]) * zs + z) * ff + cb * 128 + (lane & 15);
+#pragma unroll
+                    for (int c = 0; c < 8; c++) o[16 * c] = acc[T][c][q];
+                }
+            }
+        }
+    }
+}
+
+// Launch 2: item blockIdx.x (of the down launch's own list), 128-column blocks 4 blockIdx.y + w of hidden for wave w.  Wave w
+// first makes block w of act = silu(gate) * up for the item's tokens from launch 1's partial sums (ff <= 512: four blocks),
+// rotated into the down projection's basis; then the products over the four blocks and the output side: eo[pair][hidden].
+// grid = (bound on the items, ceil(hidden / 512)), block 256, dynamic LDS 4 XPF_LDS_WORDS.
+template <int K>
+__device__ __forceinline__ void prefill_down_exl3_kernel(const u64* __restrict__ eaddr, const u64* __restrict__ sh_addr, const u32* __restrict__ offs,
+                                                         const u32* __restrict__ list, const u32* __restrict__ items, const float* __restrict__ gup,
+                                                         float* __restrict__ eo, u32 ne, u32 k, u32 npairs, u32 NP, u32 hidden, u32 ff, u32 zs) {
+    typedef Exl3Rows<K, 4> R;
+    extern __shared__ __attribute__((aligned(16))) u32 dyn[];
+    u16* arows = (u16*) dyn;
+    u32* rings = dyn + 4 * 8 * XPF_TOK * 8;
+    u32* s_pairs = rings + 4 * R::words;
+    u32* s_rows = s_pairs + XPF_TOK;
+    float* s_max = (float*) (s_rows + XPF_TOK);
+    float* s_pre = s_max + 4 * XPF_TOK;
+    const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const u32 kbs = ff / 128;                                  // at most 4
+    u32 e;
+    const u32 nt = xpf_item(offs, list, items, blockIdx.x, ne, sh_addr != nullptr, k, npairs, s_pairs, s_rows, e);
+    if (nt == 0) return;
+    const bool two = nt > 16;
+    const u8* down = (const u8*) (e < ne ? eaddr[2ull * ne + e] : sh_addr[2]);
+    __syncthreads();
+    u32 hop[2];
+    xpf_sign_tile(lane, hop);
+    f32x4 rot[2][8];
+    float mx[2][4];
+    if (wave < kbs) {
+        const u16* suh = (const u16*) down + wave * 128 + 4 * (lane >> 4);
+        typedef u16 u16x4 __attribute__((ext_vector_type(4)));
+        float sc[8][4];
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+            const u16x4 s4 = *(const u16x4*) (suh + 16 * ks);
+#pragma unroll
+            for (int q = 0; q < 4; q++) sc[ks][q] = f16_to_f32(s4[q]);
+        }
+#pragma unroll
+        for (int T = 0; T < 2; T++) {
+            if (T == 1 && !two) break;
+            const u32 pair = s_pairs[16 * T + (lane & 15)];
+            const float* pg = gup + ((u64) pair * zs) * ff + wave * 128 + 4 * (lane >> 4);
+            const float* pu = gup + (((u64) NP + pair) * zs) * ff + wave * 128 + 4 * (lane >> 4);
+            f32x4 av[8];
+#pragma unroll
+            for (int ks = 0; ks < 8; ks++) {
+                f32x4 g = *(const f32x4*) (pg + 16 * ks), u = *(const f32x4*) (pu + 16 * ks);
+                for (u32 zz = 1; zz < zs; zz++) {
+                    g += *(const f32x4*) (pg + (u64) zz * ff + 16 * ks);
+                    u += *(const f32x4*) (pu + (u64) zz * ff + 16 * ks);
+                }
+#pragma unroll
+                for (int q = 0; q < 4; q++) av[ks][q] = (siluf_ref(g[q]) * u[q]) * sc[ks][q];
+            }
+            xpf_rotate_scaled(av, hop, rot[T], s_pre + wave * 16, lane);
+            xpf_token_max(rot[T], mx[T]);
+            if ((lane & 15) == 0) {
+#pragma unroll
+                for (int q = 0; q < 4; q++) s_max[wave * XPF_TOK + 16 * T + 4 * (lane >> 4) + q] = mx[T][q];
+            }
+        }
+    }
+    __syncthreads();
+    float inv[2][4];
+#pragma unroll
+    for (int T = 0; T < 2; T++)
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const u32 t = 16 * T + 4 * (lane >> 4) + q;
+            float m = 0.0f;
+            for (u32 w = 0; w < kbs; w++) m = fmaxf(m, s_max[w * XPF_TOK + t]);
+            float scale, iv;
+            pow2_scale_of(f32_bits(m), scale, iv);
+            inv[T][q] = iv;
+            mx[T][q] = scale * 0.08838835f;
+        }
+    if (wave < kbs) {
+        xpf_put_a_rows(arows + wave * (8 * XPF_TOK * 16), 0, rot[0], mx[0], lane);
+        if (two) xpf_put_a_rows(arows + wave * (8 * XPF_TOK * 16), 1, rot[1], mx[1], lane);
+    }
+    __syncthreads();
+    const u32 cb = 4 * blockIdx.y + wave;
+    if (cb >= hidden / 128) return;
+    const u32 wb_lds = __builtin_amdgcn_readfirstlane(lds_offset(rings + wave * R::words));
+    const u64 pitch = (u64) (hidden / 16) * EXL3_TILE_WORDS(K, false);
+    const u32* row0 = (const u32*) (down + 2 * (u64) ff + 2 * (u64) hidden + 4) + (u64) cb * 8 * EXL3_TILE_WORDS(K, false);
+    exl3_rows_issue<K, 4>(row0, pitch, lane, wb_lds);
+    f32x4 acc[2][8];
+    xpf_wave_products<K>(row0, pitch, 8 * kbs, rings + wave * R::words, wb_lds, arows, two, lane, acc);
+    const u16* svh = (const u16*) (down + 2 * (u64) ff) + cb * 128 + (lane & 15);
+    float sv[8];
+#pragma unroll
+    for (int c = 0; c < 8; c++) sv[c] = f16_to_f32(svh[16 * c]) * 0.08838835f;
+#pragma unroll
+    for (int T = 0; T < 2; T++) {
+        if (T == 1 && !two) break;
+#pragma unroll
+        for (int c = 0; c < 8; c++)
+#pragma unroll
+            for (int q = 0; q < 4; q++) acc[T][c][q] *= inv[T][q];
+        xpf_output_side(acc[T], sv, lane);
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const u32 t = 16 * T + 4 * (lane >> 4) + q;
+            if (t < nt) {
+                float* o = eo + (u64) s_pairs[t] * hidden + cb * 128 + (lane & 15);
+#pragma unroll
+                for (int c = 0; c < 8; c++) o[16 * c] = acc[T][c][q];
+            }
+        }
+    }
+}
+
+#define EXL3_PREFILL_ENTRIES(K)                                                                                                          \
+    extern "C" __global__ void __launch_bounds__(256, 2) prefill_gate_up_exl3_##K(const u64* eaddr, const u64* sh_addr, const u32* offs, const u32* list, \
+                                                                                   const u32* items, const float* x, float* gup, u32 ne, u32 k, u32 npairs, \
+                                                                                   u32 NP, u32 hidden, u32 ff) {                         \
+        prefill_gate_up_exl3_kernel<K>(eaddr, sh_addr, offs, list, items, x, gup, ne, k, npairs, NP, hidden, ff);                        \
+    }                                                                                                                                    \
+    extern "C" __global__ void __launch_bounds__(256, 2) prefill_down_exl3_##K(const u64* eaddr, const u64* sh_addr, const u32* offs, const u32* list, \
+                                                                                const u32* items, const float* gup, float* eo, u32 ne, u32 k, u32 npairs, \
+                                                                                u32 NP, u32 hidden, u32 ff, u32 zs) {                    \
+        prefill_down_exl3_kernel<K>(eaddr, sh_addr, offs, list, items, gup, eo, ne, k, npairs, NP, hidden, ff, zs);                      \
+    }
+EXL3_PREFILL_ENTRIES(1)
+EXL3_PREFILL_ENTRIES(2)
+EXL3_PREFILL_ENTRIES(3)
+EXL3_PREFILL_ENTRIES(4)
+EXL3_PREFILL_ENTRIES(5)
+EXL3_PREFILL_ENTRIES(6)
+EXL3_PREFILL_ENTRIES(7)
+EXL3_PREFILL_ENTRIES(8)

@@ -95,12 +95,12 @@ extern "C" __global__ void __launch_bounds__(256) prefill_front(const float* x, 
 // (pair = token * k + rank; the shared expert, index ne, takes the pairs npairs + token when nshared = tokens).  Also
 // cnt[token] = its number of valid experts.  The order of an expert's pairs in list[] is arbitrary; every pair owns its
 // output rows, so the results do not depend on it.  items[0] = the number of work items, items[1 + 2 i], items[2 + 2 i] =
-// (expert, first position) of item i: every run of up to PF_TOK pairs of an expert is one item of the gate/up kernel (at most
-// ne + 1 + rows / PF_TOK of them); items_d likewise with runs of up to PF_TOK_D pairs, for the down kernel.  The items that
+// (expert, first position) of item i: every run of up to unit_gu pairs of an expert is one item of the gate/up kernel (at most
+// ne + 1 + rows / unit_gu of them; PF_TOK for the int8 kernels below); items_d likewise with runs of up to unit_d pairs, for the down kernel.  The items that
 // exist come first in both lists, so the workgroups launched for the rest of the bound run at the launches' ends, out of
 // the way.  One workgroup.  grid 1, block 1024; ne <= 512.
 extern "C" __global__ void __launch_bounds__(1024) prefill_group(const u32* tidx, u32 tokens, u32 k, u32 ne, u32 nshared, u32* offs, u32* list,
-                                                                 u32* cnt, u32* items, u32* items_d) {
+                                                                 u32* cnt, u32* items, u32* items_d, u32 unit_gu, u32 unit_d) {
     __shared__ u32 s_cnt[513], s_off[514], s_fill[513], s_fill_d[513];
     const u32 tid = threadIdx.x, npairs = tokens * k, nexp = ne + 1;
     for (u32 i = tid; i < nexp; i += 1024) {
@@ -124,7 +124,7 @@ extern "C" __global__ void __launch_bounds__(1024) prefill_group(const u32* tidx
     {
         const u32 w = tid >> 6, lane = tid & 63;
         if (w < 3) {
-            const u32 unit = w == 0 ? 1u : w == 1 ? (u32) PF_TOK : (u32) PF_TOK_D;   // pairs; gate/up items; down items
+            const u32 unit = w == 0 ? 1u : w == 1 ? unit_gu : unit_d;   // pairs; gate/up items; down items
             u32 v[9], sum = 0;
 #pragma unroll
             for (int q = 0; q < 9; q++) {
@@ -156,12 +156,12 @@ extern "C" __global__ void __launch_bounds__(1024) prefill_group(const u32* tidx
     __syncthreads();
     for (u32 i = tid; i < nexp; i += 1024) {
         u32 ni = s_fill[i];
-        for (u32 t0 = 0; t0 < s_cnt[i]; t0 += PF_TOK, ni++) {
+        for (u32 t0 = 0; t0 < s_cnt[i]; t0 += unit_gu, ni++) {
             items[1 + 2 * ni] = i;
             items[2 + 2 * ni] = t0;
         }
         ni = s_fill_d[i];
-        for (u32 t0 = 0; t0 < s_cnt[i]; t0 += PF_TOK_D, ni++) {
+        for (u32 t0 = 0; t0 < s_cnt[i]; t0 += unit_d, ni++) {
             items_d[1 + 2 * ni] = i;
             items_d[2 + 2 * ni] = t0;
         }

@@ -1279,6 +1279,94 @@ def test_config4_prefill_chunk_full_size(gpu):
         assert rel_l2(got[j], acc) <= REL_L2, f"token {j}: {rel_l2(got[j], acc)}"
 
 
+@pytest.mark.parametrize("kb,tokens,hidden,ff,ne,k,shared", [
+    (3, 70, 512, 256, 8, 3, True),                 # experts with more than two items of 32, the last one ragged
+    (4, 33, 256, 512, 6, 2, False),                # an item of one token beside a full one; no shared expert
+    (2, 200, 1024, 512, 16, 4, True),
+    (5, 40, 256, 256, 6, 2, True),                 # the other rates' lane maps
+    (6, 24, 512, 256, 6, 3, True),
+    (8, 17, 256, 512, 4, 2, False),
+    (1, 50, 3072, 512, 8, 3, True),                # hidden not a multiple of 512: the last workgroup of the inputs has idle waves
+])
+def test_exl3_prefill_chunk_matches_the_oracle(gpu, kb, tokens, hidden, ff, ne, k, shared):
+    """A prefill chunk through a layer of EXL3 experts (f16 activations on the rows of the matrix instruction, the rotations on
+    the matrix cores, items of up to 32 tokens of one expert): routing ids and order bit-exact, weights within a unit in the
+    last place, every token's output within 1e-3 relative L2 of the exact oracle (forward.rs:1009-1034 a token at a time)."""
+    ty = sz.EXL3(kb)
+    rng = np.random.default_rng(kb * 1000 + tokens)
+    dbuf, stride, blobs, sh = build_layer(gpu, rng, ty, hidden, ff, ne, shared)
+    s = sz.Session(hidden, ff, ne, k, 1, 0, 8)
+    s.set_layer(0, ty, dbuf.data_ptr(), stride, ty if shared else 0, dbuf.data_ptr() + ne * stride if shared else 0)
+    x = rng.normal(size=(tokens, hidden)).astype(np.float32)
+    x[3] *= 300.0                                            # rows of very different sizes: the per-token power of two
+    x[5] *= 1e-4
+    logits = rng.normal(size=(tokens, ne)).astype(np.float32)
+    sgl = rng.normal(size=tokens).astype(np.float32)
+    dx, dl, dg = dev(gpu, x), dev(gpu, logits), dev(gpu, sgl)
+    y = gpu.zeros((tokens, hidden), dtype=gpu.float32, device="cuda")
+    print("exl3 prefill", kb, tokens, hidden, ff, flush=True)
+    s.moe_prefill_chunk(0, tokens, dx.data_ptr(), dl.data_ptr(), dg.data_ptr(), y.data_ptr())
+    gpu.cuda.synchronize()
+    got = y.cpu().numpy()
+    tidx = np.empty((tokens, k), np.uint32)
+    sz.check(sz.lib().sz_download(tidx.ctypes.data, s.prefill_buffer(2), tidx.nbytes))
+    wts = np.empty((tokens, k), np.float32)
+    sz.check(sz.lib().sz_download(wts.ctypes.data, s.prefill_buffer(3), wts.nbytes))
+    want, widx, ww = oracle_layer(ty, hidden, ff, k, blobs, sh, logits, sgl, x)
+    assert np.array_equal(tidx, widx), "expert routing must be bit-exact (ids and order)"
+    assert np.allclose(wts, ww, rtol=2e-6, atol=0)
+    assert np.all(np.isfinite(got))
+    errs = np.array([rel_l2(got[j], want[j]) for j in range(tokens)])
+    print(f"relative L2 of a token: median {np.median(errs):.3g}, worst {errs.max():.3g} (token {int(errs.argmax())})", flush=True)
+    assert errs.max() <= REL_L2
+    # twice the same bits, and a token's row does not depend on the other tokens of its chunk
+    y2 = gpu.zeros((tokens, hidden), dtype=gpu.float32, device="cuda")
+    s.moe_prefill_chunk(0, tokens, dx.data_ptr(), dl.data_ptr(), dg.data_ptr(), y2.data_ptr())
+    gpu.cuda.synchronize()
+    assert np.array_equal(bits(y2.cpu().numpy()), bits(got))
+
+
+def test_exl3_prefill_chunk_full_size(gpu):
+    """512 tokens x hidden 2048 through 512 EXL3 K = 3 experts plus the shared one, top-10 with Zipf-skewed routing (the int8
+    chunk's configuration with the verify round's experts): routing of every token bit-exact, a sample of tokens against the
+    exact oracle, every row finite and non-zero."""
+    from shadow_engine_amd import synth_device
+    torch = gpu
+    rng = np.random.default_rng(45)
+    tokens, hidden, ff, ne, k, kb = 512, 2048, 512, 512, 10, 3
+    buf, stride = synth_device.exl3_layer(torch, 4321, hidden, ff, ne, kb)
+    s = sz.Session(hidden, ff, ne, k, 1, 0, 8)
+    s.set_layer(0, sz.EXL3(kb), buf.data_ptr(), stride, sz.EXL3(kb), buf.data_ptr() + ne * stride)
+    x = rng.normal(size=(tokens, hidden)).astype(np.float32)
+    logits = synth.zipf_router_logits(rng, tokens, ne)
+    sgl = rng.normal(size=tokens).astype(np.float32)
+    dx, dl, dg = dev(gpu, x), dev(gpu, logits), dev(gpu, sgl)
+    y = gpu.zeros((tokens, hidden), dtype=gpu.float32, device="cuda")
+    s.moe_prefill_chunk(0, tokens, dx.data_ptr(), dl.data_ptr(), dg.data_ptr(), y.data_ptr())
+    gpu.cuda.synchronize()
+    got = y.cpu().numpy()
+    tidx = np.empty((tokens, k), np.uint32)
+    sz.check(sz.lib().sz_download(tidx.ctypes.data, s.prefill_buffer(2), tidx.nbytes))
+    for j in range(tokens):
+        assert np.array_equal(tidx[j], O.route(logits[j], k)[0]), f"token {j}"
+    counts = np.bincount(tidx.ravel(), minlength=ne)
+    print("distinct experts hit:", int((counts > 0).sum()), "largest group:", int(counts.max()), flush=True)
+    assert counts.max() > 64 and np.all(np.isfinite(got)) and np.all(np.abs(got).max(axis=1) > 0)
+    oty = O.exl3_type(kb)
+    shape = O.expert_shape(oty, oty, hidden, ff)
+    nb = shape.gate_bytes + shape.up_bytes + shape.down_bytes
+    worst = 0.0
+    for j in list(range(0, tokens, 47)) + [tokens - 1]:
+        ids = tidx[j]
+        host = {int(e): buf[int(e) * stride:int(e) * stride + nb].cpu().numpy() for e in list(ids) + [ne]}
+        experts = [host.get(e, host[int(ids[0])]) for e in range(ne)]
+        want, widx, _ = O.moe_token(shape, experts, k, logits[j], x[j], shape, host[ne], float(sgl[j]))
+        assert np.array_equal(widx, ids)
+        worst = max(worst, rel_l2(got[j], want))
+    print(f"worst relative L2 of a sampled token: {worst:.3g}", flush=True)
+    assert worst <= REL_L2
+
+
 def test_prefill_chunk_of_the_largest_size_equals_its_parts(gpu):
     """16384 tokens (the reference's largest staged pass, session.rs:191) in one chunk against the same tokens in chunks of
     2048 and 512: a token's result does not depend on which other tokens share its chunk (every pair owns its output row and
