@@ -254,8 +254,11 @@ def exl3_prefill(torch, sz, synth, synth_device, stream, tokens=512, bits=3):
     zs = HIDDEN // 512
     gu, dn = 2 * synth.exl3_blob_len(HIDDEN, FF, bits), synth.exl3_blob_len(FF, HIDDEN, bits)
     w.step_bytes = distinct * (gu + dn) + tokens * (2 * HIDDEN + NE) * 4
+    # gate/up: the experts' two matrices, the rows of x, the raw partial sums; act: the partial sums in, f16 operand rows out;
+    # down: the experts' third matrix, the operand rows, the pairs' rows of the result
     w.kernel_bytes = {"prefill_gate_up_exl3_%d" % bits: distinct * gu + tokens * HIDDEN * 4 + pairs * 2 * zs * FF * 4,
-                      "prefill_down_exl3_%d" % bits: distinct * dn + pairs * 2 * zs * FF * 4 + pairs * HIDDEN * 4}
+                      "prefill_act_exl3": pairs * 2 * zs * FF * 4 + pairs * FF * 2,
+                      "prefill_down_exl3_%d" % bits: distinct * dn + pairs * FF * 2 + pairs * HIDDEN * 4}
     w.dtype = "f32 accumulate over EXL3 f16 codebook weights x f16 activations (matrix cores)"
     w.describe = {"workload": "prefill chunk, %d tokens x hidden 2048 through 512 EXL3 K=%d experts + the shared one (top-10, Zipf-skewed routing, "
                               "%d distinct experts hit), f16 activations" % (tokens, bits, distinct), "rows": tokens, "resident_GB": round(buf.numel() / 1e9, 2)}

@@ -239,7 +239,9 @@ int32_t sz_copy_ranges(const uint64_t* ranges, uint32_t n, uint64_t stream);
  * gate and up, 2 the down products (EXL3 layers); 3 the gate and up rows, 4 the down rows of a GGUF layer's pairs; of the
  * head's 2-bit screen: 5 the levels, 6 their f16 scales, 7 the rows' int8 codes, 8 their scales, 9 their correction terms, 10 the
  * block maxima f32[m][vocab / 128], 11 the list of chosen blocks (count, then the blocks ascending), 12 the packed logits of the
- * listed blocks (rows 128 * min(m * k_use, vocab / 128) apart).  0 for any other `which`. */
+ * listed blocks (rows 128 * min(m * k_use, vocab / 128) apart); of the prefill chunk of EXL3 experts: 13 the partial sums of
+ * gate and up, 14 the pairs' down rows, 15 the operand rows of the down launch, 16 their factors, 17 the work items.  0 for any
+ * other `which`. */
 uint64_t sz_session_buffer(sz_session*, int32_t which);
 
 /* A whole verify round over device-resident inputs: for every layer l the MoE block on u[l][m][hidden] with rl[l][m][ne]

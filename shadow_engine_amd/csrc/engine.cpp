@@ -328,7 +328,7 @@ struct sz_session {
         DevBuf w_q2, w_sc, xq, x_sc, x_corr, bmax, seen, sel, logits;
     } hp;
     struct {
-        DevBuf xq, xd, tidx, w, cnt, offs, list, items, hq, hd, eo, gup;
+        DevBuf xq, xd, tidx, w, cnt, offs, list, items, hq, hd, eo, gup, arows, ainv;
     } pf;   // the prefill chunk's buffers, grown on demand
     void* top_host = nullptr;  // pinned host memory the top-64 merge writes to directly (8 rows of 128 words): no copy back
     bool last_fused = false;   // the last layer call left its routing in the fused layout [tidx | w | cnt]
@@ -891,7 +891,7 @@ int32_t sz_session_set_head_proxy(sz_session* s, uint32_t k_blk) {
 uint64_t sz_session_buffer(sz_session* s, int32_t which) {
     if (!s) return 0;
     const uint64_t at[] = {s->last_plan ? s->last_plan : s->plan.ptr, s->part.ptr, s->dn.ptr, s->eg.ptr, s->eo.ptr, s->hp.w_q2.ptr, s->hp.w_sc.ptr, s->hp.xq.ptr, s->hp.x_sc.ptr,
-                           s->hp.x_corr.ptr, s->hp.bmax.ptr, s->hp.sel.ptr, s->hp.logits.ptr};
+                           s->hp.x_corr.ptr, s->hp.bmax.ptr, s->hp.sel.ptr, s->hp.logits.ptr, s->pf.gup.ptr, s->pf.eo.ptr, s->pf.arows.ptr, s->pf.ainv.ptr, s->pf.items.ptr};
     return which >= 0 && which < (int32_t) (sizeof at / sizeof at[0]) ? at[which] : 0;
 }
 
@@ -1081,13 +1081,15 @@ int32_t sz_moe_prefill_chunk(sz_session* s, uint32_t l, uint32_t tokens, uint64_
     const uint64_t T = tokens, k = c.top_k, np = T * k, rows = np + (shared ? T : 0);
     auto& pb = s->pf;
     if (exl3) {
-        // EXL3 experts: f16 activations on the rows of the matrix instruction, both rotations on the matrix cores, items of up to
-        // 32 pairs (kernels/exl3.hip, "the prefill chunk of an EXL3 layer")
-        if (c.ff > 512) return fail("sz_moe_prefill_chunk: EXL3 experts of more than 512 intermediate features are not built (the down launch keeps four 128-blocks of a token)");
+        // EXL3 experts: f16 activations on the columns of the matrix instruction, the rotations on the matrix cores too, items of
+        // up to `tok` pairs (kernels/exl3.hip, "the prefill chunk of an EXL3 layer": XPF_NT, XPF_TOK, XPF_LDS_WORDS)
+        if (c.ff > 512) return fail("sz_moe_prefill_chunk: EXL3 experts of more than 512 intermediate features are not built (a workgroup keeps four 128-blocks of a token)");
         const uint32_t zs = (c.hidden / 128 + 3) / 4;
-        const uint64_t max_items = c.n_expert + 1 + rows / 32;
+        const uint32_t tok = 16 * (f.bits <= 7 ? 3 : 2), depth = f.bits <= 2 ? 8 : f.bits <= 5 ? 6 : 4;   // XPF_NT, XPF_D
+        const uint64_t max_items = c.n_expert + 1 + rows / tok;
         if (pb.tidx.need(np * 4) || pb.w.need(np * 4) || pb.cnt.need(T * 4) || pb.offs.need((c.n_expert + 2) * 4ull) || pb.list.need(rows * 4) ||
-            pb.items.need((2 + 4 * max_items) * 4) || pb.gup.need(2ull * rows * zs * c.ff * 4) || pb.eo.need(rows * c.hidden * 4))
+            pb.items.need((2 + 4 * max_items) * 4) || pb.gup.need(2ull * rows * zs * c.ff * 4) || pb.eo.need(rows * c.hidden * 4) ||
+            pb.arows.need(max_items * tok * 1024) || pb.ainv.need(max_items * tok * 4))
             return 1;
         const uint64_t sh = shared ? L.eaddr.ptr + 3ull * c.n_expert * 8 : 0, items_d = pb.items.ptr + (1 + 2 * max_items) * 4;
         {
@@ -1096,19 +1098,24 @@ int32_t sz_moe_prefill_chunk(sz_session* s, uint32_t l, uint32_t tokens, uint64_
         }
         {
             const sz_arg a[] = {P(pb.tidx.ptr), U32(tokens), U32(c.top_k), U32(c.n_expert), U32(shared ? tokens : 0), P(pb.offs.ptr), P(pb.list.ptr), P(pb.cnt.ptr),
-                                P(pb.items.ptr), P(items_d), U32(32), U32(32)};
+                                P(pb.items.ptr), P(items_d), U32(tok), U32(tok)};
             if (launch("prefill_group", 1, 1, 1, 1024, 0, stream, a)) return 1;
         }
         const uint32_t stride = (f.bits == 3 || f.bits == 4) ? 4 : (uint32_t) f.bits;
-        const uint32_t lds = 4 * (4 * 8 * 32 * 8 + 4 * (4 * 64 * stride) + 2 * 32 + 4 * 32 + 4 * 16);   // XPF_LDS_WORDS
+        const uint32_t lds = 4 * (tok / 16 * 4096 + 4 * (depth * 64 * stride) + 2 * tok + 4 * tok + tok);   // XPF_LDS_WORDS
         {
             const sz_arg a[] = {P(L.eaddr.ptr), P(sh), P(pb.offs.ptr), P(pb.list.ptr), P(pb.items.ptr), P(x), P(pb.gup.ptr), U32(c.n_expert), U32(c.top_k),
                                 U32((uint32_t) np), U32((uint32_t) rows), U32(c.hidden), U32(c.ff)};
             if (launch(("prefill_gate_up_" + tag).c_str(), (uint32_t) max_items, 2 * zs, 1, 256, lds, stream, a)) return 1;
         }
         {
-            const sz_arg a[] = {P(L.eaddr.ptr), P(sh), P(pb.offs.ptr), P(pb.list.ptr), P(items_d), P(pb.gup.ptr), P(pb.eo.ptr), U32(c.n_expert), U32(c.top_k),
-                                U32((uint32_t) np), U32((uint32_t) rows), U32(c.hidden), U32(c.ff), U32(zs)};
+            const sz_arg a[] = {P(L.eaddr.ptr), P(sh), P(pb.offs.ptr), P(pb.list.ptr), P(pb.items.ptr), P(pb.gup.ptr), P(pb.arows.ptr), P(pb.ainv.ptr), U32(c.n_expert),
+                                U32(c.top_k), U32((uint32_t) np), U32((uint32_t) rows), U32(c.hidden), U32(c.ff), U32(zs), U32(tok)};
+            if (launch("prefill_act_exl3", (uint32_t) max_items, tok / 16, 1, 256, 0, stream, a)) return 1;
+        }
+        {
+            const sz_arg a[] = {P(L.eaddr.ptr), P(sh), P(pb.offs.ptr), P(pb.list.ptr), P(pb.items.ptr), P(pb.arows.ptr), P(pb.ainv.ptr), P(pb.eo.ptr), U32(c.n_expert),
+                                U32(c.top_k), U32((uint32_t) np), U32(c.hidden), U32(c.ff)};
             if (launch(("prefill_down_" + tag).c_str(), (uint32_t) max_items, (c.hidden / 128 + 3) / 4, 1, 256, lds, stream, a)) return 1;
         }
         const sz_arg a[] = {P(y), P(pb.eo.ptr), P(pb.w.ptr), P(shared ? pb.eo.ptr + np * c.hidden * 4 : 0), P(sgl), P(pb.cnt.ptr), U32(c.hidden), U32(c.top_k)};

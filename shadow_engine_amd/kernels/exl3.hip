@@ -239,11 +239,11 @@ __device__ __forceinline__ void exl3_wave_body(const u8* __restrict__ blob, cons
 // caller: every ordinary global load whose value is still needed must have been consumed before exl3_rows_issue (a load
 // the compiler waits for later would wait for the whole burst), and a wave must pass exl3_rows_wait<K>(7) before it ends.
 // LDS layout of a tile row: decode lane L's K words start at word L * stride; K = 3 and 4 use the 16-byte lane pitch of
-// the wide loads, the others are packed.  A wave's buffer is a ring of D rows (8, or 4 where more waves must fit a CU).  Rows are requested in units: one row by
+// the wide loads, the others are packed.  A wave's buffer is a ring of D rows (8, or fewer where more waves must fit a CU).  Rows are requested in units: one row by
 // one load (K = 3, 4), two rows by one load (K = 2: a 512-byte row is half a load), one row by K one-word loads (the rest).
 template <int K, int D = 8, bool H = false>
 struct Exl3Rows {
-    static_assert(D == 4 || D == 8, "ring depths in use");
+    static_assert(D == 4 || D == 6 || D == 8, "ring depths in use");
     static constexpr int depth = D;                              // rows of the ring
     static constexpr int stride = (K == 3 || K == 4) ? 4 : K;
     static constexpr int src_words = 8 * EXL3_TILE_WORDS(K, H);  // words of a tile row of the block in memory
@@ -261,7 +261,7 @@ struct Exl3Rows {
 // row0 = the stream's first tile row (of the wave's 128-column block), pitch = words between tile rows, lds = the ring.
 template <int K, int D = 8, bool H = false>
 __device__ __forceinline__ void exl3_unit_issue(const u32* __restrict__ row0, u64 pitch, u32 r, u32 lane, u32 lds) {
-    const u32 slot = r & (D - 1);
+    const u32 slot = r % D;
     if constexpr (H) {
         typedef Exl3Rows<K, D, H> R;
 #pragma unroll
@@ -1771,21 +1771,33 @@ EXL3_LINW_ENTRIES(7)
 EXL3_LINW_ENTRIES(8)
 
 // ------------------------------------------------------------------------ the prefill chunk of an EXL3 layer (matrix cores)
-// A chunk's tokens grouped by expert (prefill_group in kernels/prefill.hip: runs of up to 32 (token, rank) pairs of one
-// expert are a work item) through gate/up and down with the item's tokens on the rows of the matrix instruction: an
-// expert's weights are decoded once for up to 32 tokens (the reference's mma_grouped_exl3_pre_K, kernels/exl3.cu:684,704,724,
-// with groups of 64, session.rs:5159-5189).  Both rotations of the format run on the matrix cores too: (x * suh) H is a
-// product with the 128 x 128 matrix of signs, whose 16 x 16 x 16 operands a lane makes from its own lane number (H[i][j] =
-// (-1)^popcount(i & j): a tile of it is a per-lane pattern times the parity of the two tile numbers), so a token's rotation
-// costs 4 matrix instructions a 128-block instead of the 130 vector instructions of the butterflies.  Inputs ride as single
-// f16 values scaled by a power of two per token and workgroup (the reference converts to f16 unscaled); weights are the
+// A chunk's tokens grouped by expert (prefill_group in kernels/prefill.hip: runs of up to XPF_TOK(K) (token, rank) pairs of
+// one expert are a work item) through gate/up, the activation and down with the item's tokens on the columns of the matrix
+// instruction: an expert's weights are decoded once for all tokens of an item (the reference's mma_grouped_exl3_pre_K,
+// kernels/exl3.cu:684,704,724, with groups of 64, session.rs:5159-5189).  The rotations of the format run on the matrix
+// cores too: H (x * suh) is a product with the 128 x 128 matrix of signs, whose 16 x 16 x 16 operands a lane makes from
+// its own lane number (H[i][j] = (-1)^popcount(i & j): a tile of it is a per-lane pattern times the parity of the two
+// tile numbers).  Every product here has the tokens on the columns (operand B, lane 16 a + n: token n, inputs 4 a .. 4 a
+// + 3) and its result on the same lanes as (token n, outputs 4 a .. 4 a + 3): a result is the next product's operand as
+// it lies, nothing is transposed.  Inputs of a rotation ride as an f16 high and an f16 low part, scaled by a power of two
+// per token; the rotated values as single f16 values (the reference converts to f16 unscaled); weights are the
 // codebook's own f16 values; sums are f32.  Against the exact arithmetic the f16 roundings of the activations cost about
-// 3e-4 relative L2 of a layer's output (bound of the path: 1e-3).
+// 4e-4 relative L2 of a layer's output (bound of the path: 1e-3).
+//
+// Three launches a layer.  1: (item, gate | up, share z of the inputs): the x rotation and the products, raw partial sums
+// to memory.  2: (item, tile of 16 tokens): the partial sums added up, the output-side transforms and scales of gate and
+// up, act = silu(gate) * up, its rotation into the down projection's basis, left as the f16 operand rows of launch 3.
+// 3: (item, four 128-column blocks of hidden): the products, the output side, the pairs' rows of the layer's result.
 
-#define XPF_TOK 32
+// Tokens of a work item: as many tiles of 16 as leave room for two workgroups' LDS on a compute unit (the operand rows of four
+// 128-blocks, 1 KiB a token, and the four waves' rings of trellis rows).
+#define XPF_NT(K) ((K) <= 7 ? 3 : 2)
+// Rows of a wave's ring: what is left of half a compute unit's LDS (rows of 256, 512, 1024 (K = 3, 4) or 256 K bytes)
+#define XPF_D(K) ((K) <= 2 ? 8 : (K) <= 5 ? 6 : 4)
+#define XPF_TOK(K) (16 * XPF_NT(K))
 
-// The lane's share of a sign tile of H for the rotation product: element q of the pair is H[16 ks + 4 a + q][16 ct + n] for
-// tile numbers of even popcount(ks & ct) (a = lane / 16, n = lane % 16); the other tiles are the negative.
+// The lane's share of a sign tile of H: element q of the pair is H[16 i + n][16 j + 4 a + q] (= H[16 j + 4 a + q][16 i + n])
+// for tile numbers of even popcount(i & j) (a = lane / 16, n = lane % 16); the other tiles are the negative.
 __device__ __forceinline__ void xpf_sign_tile(u32 lane, u32 (&hop)[2]) {
     const u32 n = lane & 15, a = lane >> 4;
     u32 h[4];
@@ -1795,8 +1807,10 @@ __device__ __forceinline__ void xpf_sign_tile(u32 lane, u32 (&hop)[2]) {
     hop[1] = h[2] | (h[3] << 16);
 }
 
-// rot[ct][q] = sum over the 128 inputs i of v[token][i] H[i][16 ct + n] for token 4 a + q of the tile: v comes as load4(ks) =
-// the lane's token's (lane % 16) inputs 16 ks + 4 a .. + 3 (already times the input scales), rounded to f16 here.
+// rot[ct][q] = sum over the 128 inputs i of H[16 ct + 4 a + q][i] v[i] for the lane's token (n = lane % 16 of the tile): v
+// comes as load4(ks) = the token's inputs 16 ks + 4 a .. + 3 (already times the input scales and the token's power of two).
+// An input goes in as an f16 high and an f16 low part (22 bits of it; the signs are exact, the sums f32): the rotation
+// itself adds no rounding that matters.
 template <class F>
 __device__ __forceinline__ void xpf_rotate_tile(F&& load4, const u32 (&hop)[2], f32x4 (&rot)[8]) {
 #pragma unroll
@@ -1807,78 +1821,62 @@ __device__ __forceinline__ void xpf_rotate_tile(F&& load4, const u32 (&hop)[2], 
     for (int ks = 0; ks < 8; ks++) {
         const f32x4 v = load4(ks);
         const f16x4 av = {(_Float16) v[0], (_Float16) v[1], (_Float16) v[2], (_Float16) v[3]};
+        const f16x4 al = {(_Float16) (v[0] - (float) av[0]), (_Float16) (v[1] - (float) av[1]), (_Float16) (v[2] - (float) av[2]), (_Float16) (v[3] - (float) av[3])};
 #pragma unroll
         for (int ct = 0; ct < 8; ct++) {
             const bool neg = __builtin_popcount(ks & ct) & 1;
-            rot[ct] = __builtin_amdgcn_mfma_f32_16x16x16f16(av, __builtin_bit_cast(f16x4, neg ? hn : hp), rot[ct], 0, 0, 0);
+            rot[ct] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, neg ? hn : hp), av, rot[ct], 0, 0, 0);
+            rot[ct] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, neg ? hn : hp), al, rot[ct], 0, 0, 0);
         }
     }
 }
 
-// The power of two that takes the largest magnitude of the lane's token's (lane % 16) 128 inputs to [2^14, 2^15), so that they
-// round to f16 without overflow or loss of small values, and its inverse: v = the lane's 32 of them (the other 96 are in
-// lanes + 16, + 32, + 48).
-__device__ __forceinline__ void xpf_input_scale(const f32x4 (&v)[8], u32 lane, float& scale, float& inv) {
+// The largest magnitude of the lane's token's 128 values: the lane's 32 of them, then the lanes + 16, + 32, + 48.
+__device__ __forceinline__ float xpf_token_max(const f32x4 (&v)[8], u32 lane) {
     float m = 0.0f;
 #pragma unroll
     for (int ks = 0; ks < 8; ks++)
 #pragma unroll
         for (int q = 0; q < 4; q++) m = fmaxf(m, __builtin_fabsf(v[ks][q]));
     m = fmaxf(m, lane_xor<16>(m, lane));
-    m = fmaxf(m, lane_xor<32>(m, lane));
-    pow2_scale_of(f32_bits(m), scale, inv);
+    return fmaxf(m, lane_xor<32>(m, lane));
 }
 
-// The largest magnitude of each of the lane's four tokens (4 a + q) over the tile's 128 rotated values: over the lane's 8
-// column tiles, then over the 16 lanes of its row.
-__device__ __forceinline__ void xpf_token_max(const f32x4 (&rot)[8], float (&mx)[4]) {
+// A 128-block of the lane's token through H, its values brought into f16's range for the product by the token's own power
+// of two and back afterwards (exact both ways): rot = H v.
+__device__ __forceinline__ void xpf_rotate_scaled(const f32x4 (&v)[8], const u32 (&hop)[2], f32x4 (&rot)[8], u32 lane) {
+    float scale, inv;
+    pow2_scale_of(f32_bits(xpf_token_max(v, lane)), scale, inv);
+    xpf_rotate_tile([&](int ks) { return v[ks] * scale; }, hop, rot);
 #pragma unroll
-    for (int q = 0; q < 4; q++) {
-        float m = 0.0f;
+    for (int ct = 0; ct < 8; ct++) rot[ct] *= inv;
+}
+
+// The operand rows of the products.  A token tile's rows: [tile row i of the item's up to 32 (block * 8 + ct)][token n][16
+// values in the order the decode lanes take them], 512 bytes a tile row; the tiles of an item follow each other.  The lane
+// holds the values 4 a + q of tile row ct of its token: slots 8 (a & 1) + 2 (a >> 1) + {0, 1} and + 4 of that (exl3_aslot).
+// rot must be bounded by 2^22 (inputs scaled to below 2^15, 128 terms): the stored value is f16(rot / 128).
+#define XPF_TILE_U16 (32 * 256)      // u16 of a token tile's operand rows (four 128-blocks)
+__device__ __forceinline__ void xpf_put_rows(u16* tile, u32 block, const f32x4 (&rot)[8], u32 lane) {
+    const u32 n = lane & 15, a = lane >> 4;
+    u32* at = (u32*) (tile + (block * 8) * 256 + n * 16 + 8 * (a & 1) + 2 * (a >> 1));
 #pragma unroll
-        for (int ct = 0; ct < 8; ct++) m = fmaxf(m, __builtin_fabsf(rot[ct][q]));
-        m = fmaxf(m, bits_f32(__builtin_amdgcn_update_dpp(0u, f32_bits(m), 0xb1, 0xf, 0xf, true)));    // quad_perm [1,0,3,2]
-        m = fmaxf(m, bits_f32(__builtin_amdgcn_update_dpp(0u, f32_bits(m), 0x4e, 0xf, 0xf, true)));    // quad_perm [2,3,0,1]
-        m = fmaxf(m, bits_f32(__builtin_amdgcn_update_dpp(0u, f32_bits(m), 0x124, 0xf, 0xf, true)));   // row_ror:4
-        m = fmaxf(m, bits_f32(__builtin_amdgcn_update_dpp(0u, f32_bits(m), 0x128, 0xf, 0xf, true)));   // row_ror:8
-        mx[q] = m;
+    for (int ct = 0; ct < 8; ct++) {
+        const f16x2 lo = {(_Float16) (rot[ct][0] * 0.0078125f), (_Float16) (rot[ct][1] * 0.0078125f)};
+        const f16x2 hi = {(_Float16) (rot[ct][2] * 0.0078125f), (_Float16) (rot[ct][3] * 0.0078125f)};
+        at[ct * 128] = __builtin_bit_cast(u32, lo);
+        at[ct * 128 + 2] = __builtin_bit_cast(u32, hi);
     }
 }
+// what undoes the 1 / 128 of the stored values and applies the transform's 1 / sqrt(128)
+#define XPF_UNSCALE 11.3137085f
 
-// A tile's rotation with its inputs brought into f16's range first: every token's inputs times its own power of two, the
-// transform, and the rotated values times the inverse (exact both ways).  pre: 16 floats of the wave's own LDS.
-__device__ __forceinline__ void xpf_rotate_scaled(f32x4 (&v)[8], const u32 (&hop)[2], f32x4 (&rot)[8], float* pre, u32 lane) {
-    float scale, inv;
-    xpf_input_scale(v, lane, scale, inv);
-    if (lane < 16) pre[lane] = inv;
-    xpf_rotate_tile([&](int ks) { return v[ks] * scale; }, hop, rot);
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
-    __builtin_amdgcn_wave_barrier();
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-    const f32x4 iv = *(const f32x4*) (pre + 4 * (lane >> 4));   // of the lane's tokens 4 a + q
-#pragma unroll
-    for (int ct = 0; ct < 8; ct++) rot[ct] *= iv;
-    __builtin_amdgcn_wave_barrier();                             // the strip is free for the next tile
-}
-
-// The tile's rotated values as A rows of the products: f16(rot * sc[q]) at arows[(ct * XPF_TOK + 16 T + 4 a + q) * 16 + slot of n]
-// (tile row ct of the 128-block, A row = the token's place in the item).
-__device__ __forceinline__ void xpf_put_a_rows(u16* arows, u32 T, const f32x4 (&rot)[8], const float (&sc)[4], u32 lane) {
-    const u32 n = lane & 15, a = lane >> 4;
-    u16* at = arows + (16 * T + 4 * a) * 16 + exl3_aslot(n);
-#pragma unroll
-    for (int ct = 0; ct < 8; ct++)
-#pragma unroll
-        for (int q = 0; q < 4; q++) at[(ct * XPF_TOK + q) * 16] = __builtin_bit_cast(u16, (_Float16) (rot[ct][q] * sc[q]));
-}
-
-// The products of one wave: `nrows` tile rows of its 128-column block (the stream starts at row0, its first rows requested
-// by exl3_mma_rows_start) against the A rows at xa (tile row i at xa + i * XPF_TOK * 16, A row = token) for one or two
-// token tiles; acc[T][c] as exl3_wave_mma's (row 4 a + q = token 16 T + 4 a + q).
-template <int K>
-__device__ __forceinline__ void xpf_wave_products(const u32* __restrict__ row0, u64 pitch, u32 nrows, const u32* wb, u32 lds, const u16* xa, bool two,
-                                                  u32 lane, f32x4 (&acc)[2][8]) {
-    constexpr int D = 4;
+// The products of one wave: `nrows` tile rows of its 128-column block (the stream starts at row0, its first rows already
+// requested) against the operand rows of NT token tiles at xa; acc[T][c][q] = output 16 c + 4 a + q of token 16 T + n.
+template <int K, int NT>
+__device__ __forceinline__ void xpf_wave_products_of(const u32* __restrict__ row0, u64 pitch, u32 nrows, const u32* wb, u32 lds, const u16* xa, u32 lane,
+                                                     f32x4 (&acc)[XPF_NT(K)][8]) {
+    constexpr int D = XPF_D(K);
     typedef Exl3Rows<K, D> R;
     constexpr int stride = R::stride, ur = R::unit_rows;
     constexpr bool one_shift = 16 + 3 * K <= 32;
@@ -1894,14 +1892,14 @@ __device__ __forceinline__ void xpf_wave_products(const u32* __restrict__ row0, 
     window((t0 + 4) * K, om1, op1, sh1);
     if constexpr (!one_shift) window((t0 + 2) * K, om0, op0, sh0);
 #pragma unroll
-    for (int T = 0; T < 2; T++)
+    for (int T = 0; T < NT; T++)
 #pragma unroll
         for (int c = 0; c < 8; c++) acc[T][c] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     const u16* xa0 = xa + n16 * 16 + 4 * a;
 #pragma unroll 1
     for (u32 i = 0; i < nrows; i++) {
         exl3_rows_wait<K, D>(i + D > nrows ? i + D - nrows : 0);
-        const u32* row = wb + (i & (D - 1)) * R::row_words;
+        const u32* row = wb + (i % D) * R::row_words;
         u32 w1[8][2], w0[8][2];
 #pragma unroll
         for (int c = 0; c < 8; c++) {
@@ -1913,14 +1911,13 @@ __device__ __forceinline__ void xpf_wave_products(const u32* __restrict__ row0, 
             }
         }
         typedef u32 u32x2 __attribute__((ext_vector_type(2)));
-        const u32x2 xv0 = *(const u32x2*) (xa0 + i * (XPF_TOK * 16));
-        u32x2 xv1 = *(const u32x2*) (xa0 + i * (XPF_TOK * 16) + 16 * 16);
-        if (!two) xv1 = u32x2{0u, 0u};
+        f16x4 xv[NT];
+#pragma unroll
+        for (int T = 0; T < NT; T++) xv[T] = __builtin_bit_cast(f16x4, *(const u32x2*) (xa0 + T * XPF_TILE_U16 + i * 256));
         if ((i + 1) % ur == 0 && i + D + 1 - ur < nrows) {
             __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): the row's words are in registers, its slot can take the row D further on
             exl3_unit_issue<K, D>(row0, pitch, i + D + 1 - ur, lane, lds);
         }
-        const f16x4 av0 = __builtin_bit_cast(f16x4, xv0), av1 = __builtin_bit_cast(f16x4, xv1);
 #pragma unroll
         for (int c = 0; c < 8; c++) {
             const u32 hi = __builtin_amdgcn_alignbit(w1[c][0], w1[c][1], sh1);
@@ -1936,16 +1933,32 @@ __device__ __forceinline__ void xpf_wave_products(const u32* __restrict__ row0, 
             const u32 s2 = __builtin_amdgcn_ubfe(hi, K, 16), s3 = hi & 0xffffu;
             const f16x2 b01 = exl3_cb2_pair(s0, s1), b23 = exl3_cb2_pair(s2, s3);
             const f16x4 bv = {b01[0], b01[1], b23[0], b23[1]};
-            acc[0][c] = __builtin_amdgcn_mfma_f32_16x16x16f16(av0, bv, acc[0][c], 0, 0, 0);
-            if (two) acc[1][c] = __builtin_amdgcn_mfma_f32_16x16x16f16(av1, bv, acc[1][c], 0, 0, 0);
+#pragma unroll
+            for (int T = 0; T < NT; T++) acc[T][c] = __builtin_amdgcn_mfma_f32_16x16x16f16(bv, xv[T], acc[T][c], 0, 0, 0);
         }
     }
 }
 
-// The output side of a wave's block: out[c][q] (column 16 c + n of the lane's four tokens 4 a + q of one tile) through the
-// 128-point transform over the columns (three stages over c in registers, four over the lanes of the row of 16) times the
-// output scales sv[c] (column 16 c + n), the 1/sqrt(128) included.
-__device__ __forceinline__ void xpf_output_side(f32x4 (&v)[8], const float (&sv)[8], u32 lane) {
+// One loop for every number of token tiles: the choice is made once, outside the loop.
+template <int K>
+__device__ __forceinline__ void xpf_wave_products(const u32* __restrict__ row0, u64 pitch, u32 nrows, const u32* wb, u32 lds, const u16* xa, u32 ntiles,
+                                                  u32 lane, f32x4 (&acc)[XPF_NT(K)][8]) {
+    if (ntiles == 1) xpf_wave_products_of<K, 1>(row0, pitch, nrows, wb, lds, xa, lane, acc);
+    else if (ntiles == 2) xpf_wave_products_of<K, 2>(row0, pitch, nrows, wb, lds, xa, lane, acc);
+    else if constexpr (XPF_NT(K) >= 3) xpf_wave_products_of<K, 3>(row0, pitch, nrows, wb, lds, xa, lane, acc);
+}
+
+// The output side of a wave's block for the lane's token: v[c][q] = output 16 c + 4 a + q goes through the 128-point
+// transform.  Five of its seven stages are between the lane's own registers; the two over the lane number's bits 4 and 5 are
+// swaps of register halves between the lanes (one swap serves two registers), after which the lane holds OTHER outputs of
+// its token: register c, element q is output xpf_out_col(c, lane) + q.
+__device__ __forceinline__ u32 xpf_out_col(u32 c, u32 lane) { return 64 * (c >> 2) + 32 * ((lane >> 4) & 1) + 16 * (lane >> 5) + 8 * (c & 1) + 4 * ((c >> 1) & 1); }
+__device__ __forceinline__ void xpf_output_side(f32x4 (&v)[8]) {
+#pragma unroll
+    for (int c = 0; c < 8; c++) {
+        const float t0 = v[c][0] + v[c][1], t1 = v[c][0] - v[c][1], t2 = v[c][2] + v[c][3], t3 = v[c][2] - v[c][3];
+        v[c] = f32x4{t0 + t2, t1 + t3, t0 - t2, t1 - t3};
+    }
 #pragma unroll
     for (int h = 1; h < 8; h <<= 1)
 #pragma unroll
@@ -1955,28 +1968,40 @@ __device__ __forceinline__ void xpf_output_side(f32x4 (&v)[8], const float (&sv)
                 v[c] = s;
                 v[c + h] = d;
             }
+    // lane bit 5 (output bit 3): the upper half of register c and the lower half of register c + 1 change places; then both lanes
+    // of a pair hold the two ends of one butterfly.  Register c keeps the sum (bit 3 clear), c + 1 the difference; the lane's
+    // bit 5 now says which of the two registers' outputs (output bit 4) it holds.
 #pragma unroll
-    for (int c = 0; c < 8; c++)
+    for (int c = 0; c < 8; c += 2)
 #pragma unroll
         for (int q = 0; q < 4; q++) {
-            float x = v[c][q];
-            { const float p = lane_xor<1>(x, lane); x = __builtin_fmaf(x, bits_f32(0x3f800000u | ((lane & 1) ? 0x80000000u : 0u)), p); }
-            { const float p = lane_xor<2>(x, lane); x = __builtin_fmaf(x, bits_f32(0x3f800000u | ((lane & 2) ? 0x80000000u : 0u)), p); }
-            { const float p = lane_xor<4>(x, lane); x = __builtin_fmaf(x, bits_f32(0x3f800000u | ((lane & 4) ? 0x80000000u : 0u)), p); }
-            { const float p = lane_xor<8>(x, lane); x = __builtin_fmaf(x, bits_f32(0x3f800000u | ((lane & 8) ? 0x80000000u : 0u)), p); }
-            v[c][q] = x * sv[c];
+            const auto r = __builtin_amdgcn_permlane32_swap(f32_bits(v[c][q]), f32_bits(v[c + 1][q]), false, false);
+            v[c][q] = bits_f32(r[0]) + bits_f32(r[1]);
+            v[c + 1][q] = bits_f32(r[0]) - bits_f32(r[1]);
+        }
+    // lane bit 4 (output bit 2) with the registers c and c + 2 (output bit 5) likewise
+#pragma unroll
+    for (int c = 0; c < 8; c++)
+        if (!(c & 2)) {
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const auto r = __builtin_amdgcn_permlane16_swap(f32_bits(v[c][q]), f32_bits(v[c + 2][q]), false, false);
+                v[c][q] = bits_f32(r[0]) + bits_f32(r[1]);
+                v[c + 2][q] = bits_f32(r[0]) - bits_f32(r[1]);
+            }
         }
 }
 
-// Shared set-up of the two launches: the item, its pairs and rows.  Returns the number of the item's pairs (0: no such item).
+// Shared set-up of the launches: the item, its pairs and rows (tok = the most pairs of an item).  Returns the number of the
+// item's pairs (0: no such item).
 __device__ __forceinline__ u32 xpf_item(const u32* __restrict__ offs, const u32* __restrict__ list, const u32* __restrict__ items, u32 item, u32 ne, bool has_shared,
-                                        u32 k, u32 npairs, u32* s_pairs, u32* s_rows, u32& e) {
+                                        u32 k, u32 npairs, u32 tok, u32* s_pairs, u32* s_rows, u32& e) {
     if (item >= items[0]) return 0;
     e = items[1 + 2 * item];
     const u32 t0 = items[2 + 2 * item];
     if (e == ne && !has_shared) return 0;
-    const u32 first = offs[e], nt = min((u32) XPF_TOK, offs[e + 1] - first - t0);
-    if (threadIdx.x < XPF_TOK) {
+    const u32 first = offs[e], nt = min(tok, offs[e + 1] - first - t0);
+    if (threadIdx.x < tok) {
         const u32 p = list[first + t0 + min(threadIdx.x, nt - 1)];   // a place past the item's end repeats its last pair: loads stay in bounds, results are dropped
         s_pairs[threadIdx.x] = p;
         s_rows[threadIdx.x] = p < npairs ? p / k : p - npairs;
@@ -1984,52 +2009,48 @@ __device__ __forceinline__ u32 xpf_item(const u32* __restrict__ offs, const u32*
     return nt;
 }
 
-// LDS of a workgroup of the two launches, in words: the A rows of four 128-blocks (32 tokens each), the four waves' rings,
-// the item's pairs and rows, the waves' token maxima, the waves' strips of 16 input scales.
-#define XPF_LDS_WORDS(ring) (4 * 8 * XPF_TOK * 8 + 4 * (ring) + 2 * XPF_TOK + 4 * XPF_TOK + 4 * 16)
+// LDS of a workgroup of launches 1 and 3, in words: the operand rows of the item's token tiles, the four waves' rings, the
+// item's pairs and rows, the waves' token maxima, the tokens' factors.
+#define XPF_LDS_WORDS(ring, tok) ((tok) / 16 * (XPF_TILE_U16 / 2) + 4 * (ring) + 2 * (tok) + 4 * (tok) + (tok))
 
 // Launch 1: item blockIdx.x, sel = blockIdx.y / zs (gate, up), z = blockIdx.y % zs: the inputs' 128-blocks 4 z .. 4 z + 3.
 // Wave w rotates block 4 z + w of the item's tokens, then takes the 128-column blocks w, w + 4, .. of ff over the four input
-// blocks; partial sums gup[((sel * NP + pair) * zs + z)][ff], already through the output-side transform and scales (NP =
-// npairs + the shared expert's rows).  grid = (bound on the items, 2 zs), block 256, dynamic LDS 4 XPF_LDS_WORDS.
+// blocks; raw partial sums gup[((sel * NP + pair) * zs + z)][ff] (NP = npairs + the shared expert's rows): the output side
+// is launch 2's.  grid = (bound on the items, 2 zs), block 256, dynamic LDS 4 XPF_LDS_WORDS.
 template <int K>
 __device__ __forceinline__ void prefill_gate_up_exl3_kernel(const u64* __restrict__ eaddr, const u64* __restrict__ sh_addr, const u32* __restrict__ offs,
                                                             const u32* __restrict__ list, const u32* __restrict__ items, const float* __restrict__ x,
                                                             float* __restrict__ gup, u32 ne, u32 k, u32 npairs, u32 NP, u32 hidden, u32 ff) {
-    typedef Exl3Rows<K, 4> R;
+    typedef Exl3Rows<K, XPF_D(K)> R;
+    constexpr u32 TOK = XPF_TOK(K);
     extern __shared__ __attribute__((aligned(16))) u32 dyn[];
-    u16* arows = (u16*) dyn;                                  // [block of the four][tile row][token][16]
-    u32* rings = dyn + 4 * 8 * XPF_TOK * 8;
+    u16* arows = (u16*) dyn;                                  // [token tile][block of the four][tile row][token][16]
+    u32* rings = dyn + XPF_NT(K) * (XPF_TILE_U16 / 2);
     u32* s_pairs = rings + 4 * R::words;
-    u32* s_rows = s_pairs + XPF_TOK;
-    float* s_max = (float*) (s_rows + XPF_TOK);               // [wave][token]
-    float* s_pre = s_max + 4 * XPF_TOK;                       // [wave][16]
+    u32* s_rows = s_pairs + TOK;
+    float* s_max = (float*) (s_rows + TOK);                   // [wave][token]
+    float* s_inv = s_max + 4 * TOK;                           // [token]
     const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const u32 kbs = hidden / 128, zs = (kbs + 3) / 4, sel = blockIdx.y / zs, z = blockIdx.y - sel * zs;
     u32 e;
-    const u32 nt = xpf_item(offs, list, items, blockIdx.x, ne, sh_addr != nullptr, k, npairs, s_pairs, s_rows, e);
+    const u32 nt = xpf_item(offs, list, items, blockIdx.x, ne, sh_addr != nullptr, k, npairs, TOK, s_pairs, s_rows, e);
     if (nt == 0) return;
-    const bool two = nt > 16;
+    const u32 ntiles = (nt + 15) / 16;
     const u8* bp = (const u8*) (e < ne ? eaddr[(u64) sel * ne + e] : sh_addr[sel]);
     const u32 kb = 4 * z + wave, nkb = min(4u, kbs - 4 * z);
     __syncthreads();                                          // the item's pairs and rows are written
-    u32 hop[2];
-    xpf_sign_tile(lane, hop);
-    f32x4 rot[2][8];
-    float mx[2][4];
+    typedef u16 u16x4 __attribute__((ext_vector_type(4)));
+    float sc[8][4];
     if (wave < nkb) {
+        // the largest input of every token over the block: the token's power of two must be one for the workgroup's four blocks
         const u16* suh = (const u16*) bp + kb * 128 + 4 * (lane >> 4);
-        typedef u16 u16x4 __attribute__((ext_vector_type(4)));
-        float sc[8][4];
 #pragma unroll
         for (int ks = 0; ks < 8; ks++) {
             const u16x4 s4 = *(const u16x4*) (suh + 16 * ks);
 #pragma unroll
             for (int q = 0; q < 4; q++) sc[ks][q] = f16_to_f32(s4[q]);
         }
-#pragma unroll
-        for (int T = 0; T < 2; T++) {
-            if (T == 1 && !two) break;
+        for (u32 T = 0; T < ntiles; T++) {
             const float* xr = x + (u64) s_rows[16 * T + (lane & 15)] * hidden + kb * 128 + 4 * (lane >> 4);
             f32x4 xv[8];
 #pragma unroll
@@ -2038,176 +2059,195 @@ __device__ __forceinline__ void prefill_gate_up_exl3_kernel(const u64* __restric
 #pragma unroll
                 for (int q = 0; q < 4; q++) xv[ks][q] *= sc[ks][q];
             }
-            xpf_rotate_scaled(xv, hop, rot[T], s_pre + wave * 16, lane);
-            xpf_token_max(rot[T], mx[T]);
-            if ((lane & 15) == 0) {
-#pragma unroll
-                for (int q = 0; q < 4; q++) s_max[wave * XPF_TOK + 16 * T + 4 * (lane >> 4) + q] = mx[T][q];
-            }
+            const float m = xpf_token_max(xv, lane);
+            if (lane < 16) s_max[wave * TOK + 16 * T + lane] = m;
         }
     }
     __syncthreads();
-    // one power of two a token for the workgroup's four blocks; the lane's tokens 16 T + 4 a + q
-    float inv[2][4];
-#pragma unroll
-    for (int T = 0; T < 2; T++)
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const u32 t = 16 * T + 4 * (lane >> 4) + q;
+    if (wave < nkb) {
+        u32 hop[2];
+        xpf_sign_tile(lane, hop);
+        for (u32 T = 0; T < ntiles; T++) {
+            const u32 t = 16 * T + (lane & 15);
             float m = 0.0f;
-            for (u32 w = 0; w < nkb; w++) m = fmaxf(m, s_max[w * XPF_TOK + t]);
+            for (u32 w = 0; w < nkb; w++) m = fmaxf(m, s_max[w * TOK + t]);
             float scale, iv;
             pow2_scale_of(f32_bits(m), scale, iv);
-            inv[T][q] = iv;
-            mx[T][q] = scale * 0.08838835f;                   // the factor of the stored values: the power of two and the transform's 1/sqrt(128)
+            if (wave == 0 && lane < 16) s_inv[t] = iv * XPF_UNSCALE;
+            const float* xr = x + (u64) s_rows[t] * hidden + kb * 128 + 4 * (lane >> 4);   // the second read comes from the caches
+            f32x4 rot[8];
+            xpf_rotate_tile(
+                [&](int ks) {
+                    f32x4 v = *(const f32x4*) (xr + 16 * ks);
+#pragma unroll
+                    for (int q = 0; q < 4; q++) v[q] = (v[q] * sc[ks][q]) * scale;
+                    return v;
+                },
+                hop, rot);
+            xpf_put_rows(arows + T * XPF_TILE_U16, wave, rot, lane);
         }
-    if (wave < nkb) {
-        xpf_put_a_rows(arows + wave * (8 * XPF_TOK * 16), 0, rot[0], mx[0], lane);
-        if (two) xpf_put_a_rows(arows + wave * (8 * XPF_TOK * 16), 1, rot[1], mx[1], lane);
     }
     __syncthreads();
     const u32 wb_lds = __builtin_amdgcn_readfirstlane(lds_offset(rings + wave * R::words));
     const u64 pitch = (u64) (ff / 16) * EXL3_TILE_WORDS(K, false);
     for (u32 cb = wave; cb < ff / 128; cb += 4) {
         const u32* row0 = (const u32*) (bp + 2 * (u64) hidden + 2 * (u64) ff + 4) + ((u64) (4 * z) * 8 * (ff / 16) + cb * 8) * EXL3_TILE_WORDS(K, false);
-        exl3_rows_issue<K, 4>(row0, pitch, lane, wb_lds);     // a stream has at least 8 rows
-        f32x4 acc[2][8];
-        xpf_wave_products<K>(row0, pitch, 8 * nkb, rings + wave * R::words, wb_lds, arows, two, lane, acc);
-        const u16* svh = (const u16*) (bp + 2 * (u64) hidden) + cb * 128 + (lane & 15);
-        float sv[8];
+        exl3_rows_issue<K, XPF_D(K)>(row0, pitch, lane, wb_lds);     // a stream has at least 8 rows
+        f32x4 acc[XPF_NT(K)][8];
+        xpf_wave_products<K>(row0, pitch, 8 * nkb, rings + wave * R::words, wb_lds, arows, ntiles, lane, acc);
 #pragma unroll
-        for (int c = 0; c < 8; c++) sv[c] = f16_to_f32(svh[16 * c]) * 0.08838835f;
+        for (int T = 0; T < XPF_NT(K); T++) {
+            if ((u32) T >= ntiles) break;
+            const u32 t = 16 * T + (lane & 15);
+            const float iv = s_inv[t];
+            if (t < nt) {
+                float* o = gup + (((u64) sel * NP + s_pairs[t]) * zs + z) * ff + cb * 128 + 4 * (lane >> 4);
 #pragma unroll
-        for (int T = 0; T < 2; T++) {
-            if (T == 1 && !two) break;
-#pragma unroll
-            for (int c = 0; c < 8; c++)
-#pragma unroll
-                for (int q = 0; q < 4; q++) acc[T][c][q] *= inv[T][q];
-            xpf_output_side(acc[T], sv, lane);
-#pragma unroll
-            for (int q = 0; q < 4; q++) {
-                const u32 t = 16 * T + 4 * (lane >> 4) + q;
-                if (t < nt) {
-                    float* o = gup + (((u64) sel * NP + s_pairs[t]) * zs + z) * ff + cb * 128 + (lane & 15);
-#pragma unroll
-                    for (int c = 0; c < 8; c++) o[16 * c] = acc[T][c][q];
-                }
+                for (int c = 0; c < 8; c++) *(f32x4*) (o + 16 * c) = acc[T][c] * iv;
             }
         }
     }
 }
 
-// Launch 2: item blockIdx.x (of the down launch's own list), 128-column blocks 4 blockIdx.y + w of hidden for wave w.  Wave w
-// first makes block w of act = silu(gate) * up for the item's tokens from launch 1's partial sums (ff <= 512: four blocks),
-// rotated into the down projection's basis; then the products over the four blocks and the output side: eo[pair][hidden].
-// grid = (bound on the items, ceil(hidden / 512)), block 256, dynamic LDS 4 XPF_LDS_WORDS.
+// Launch 2 (one kernel for every rate): tile blockIdx.y (16 tokens) of item blockIdx.x.  Wave w takes block w of ff (ff <=
+// 512: four blocks): adds up launch 1's partial sums of gate and up, puts both through their output sides (transform, output
+// scales), act = silu(gate) * up times the down projection's input scales, rotated, and leaves it as operand rows for
+// launch 3: arows[item * tok / 16 + tile] = a token tile's rows (XPF_TILE_U16), ainv[item * tok + token] = what undoes the
+// token's power of two.  grid = (bound on the items, tok / 16), block 256.
+extern "C" __global__ void __launch_bounds__(256, 2) prefill_act_exl3(const u64* eaddr, const u64* sh_addr, const u32* offs, const u32* list, const u32* items,
+                                                                      const float* gup, u16* arows, float* ainv, u32 ne, u32 k, u32 npairs, u32 NP,
+                                                                      u32 hidden, u32 ff, u32 zs, u32 tok) {
+    __shared__ u32 s_pairs[64], s_rows[64];
+    __shared__ float s_max[4 * 16];
+    const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const u32 kbs = ff / 128, T = blockIdx.y;                  // kbs: at most 4
+    u32 e;
+    const u32 nt = xpf_item(offs, list, items, blockIdx.x, ne, sh_addr != nullptr, k, npairs, tok, s_pairs, s_rows, e);
+    if (16 * T >= nt) return;
+    __syncthreads();
+    const u8* bg = (const u8*) (e < ne ? eaddr[e] : sh_addr[0]);
+    const u8* bu = (const u8*) (e < ne ? eaddr[(u64) ne + e] : sh_addr[1]);
+    const u8* bd = (const u8*) (e < ne ? eaddr[2ull * ne + e] : sh_addr[2]);
+    typedef u16 u16x4 __attribute__((ext_vector_type(4)));
+    u32 hop[2];
+    xpf_sign_tile(lane, hop);
+    f32x4 act[8];
+    float m = 0.0f;
+    if (wave < kbs) {
+        const u32 pair = s_pairs[16 * T + (lane & 15)], at = wave * 128 + 4 * (lane >> 4);
+        const float* pg = gup + ((u64) pair * zs) * ff + at;
+        const float* pu = gup + (((u64) NP + pair) * zs) * ff + at;
+        f32x4 g[8], u[8];
+#pragma unroll
+        for (int ks = 0; ks < 8; ks++) {
+            g[ks] = *(const f32x4*) (pg + 16 * ks);
+            u[ks] = *(const f32x4*) (pu + 16 * ks);
+        }
+        for (u32 zz = 1; zz < zs; zz++)
+#pragma unroll
+            for (int ks = 0; ks < 8; ks++) {
+                g[ks] += *(const f32x4*) (pg + (u64) zz * ff + 16 * ks);
+                u[ks] += *(const f32x4*) (pu + (u64) zz * ff + 16 * ks);
+            }
+        f32x4 gr[8];
+        xpf_rotate_scaled(g, hop, gr, lane);
+        xpf_rotate_scaled(u, hop, g, lane);                    // g: the rotated up from here on
+        const u16* svg = (const u16*) (bg + 2 * (u64) hidden) + at;
+        const u16* svu = (const u16*) (bu + 2 * (u64) hidden) + at;
+        const u16* suh = (const u16*) bd + at;
+#pragma unroll
+        for (int ct = 0; ct < 8; ct++) {
+            const u16x4 a4 = *(const u16x4*) (svg + 16 * ct), b4 = *(const u16x4*) (svu + 16 * ct), c4 = *(const u16x4*) (suh + 16 * ct);
+#pragma unroll
+            for (int q = 0; q < 4; q++) {
+                const float gate = gr[ct][q] * (f16_to_f32(a4[q]) * 0.08838835f), up = g[ct][q] * (f16_to_f32(b4[q]) * 0.08838835f);
+                act[ct][q] = (siluf_ref(gate) * up) * f16_to_f32(c4[q]);
+            }
+        }
+        m = xpf_token_max(act, lane);
+        if (lane < 16) s_max[wave * 16 + lane] = m;
+    }
+    __syncthreads();
+    if (wave >= kbs) return;
+    m = 0.0f;
+    for (u32 w = 0; w < kbs; w++) m = fmaxf(m, s_max[w * 16 + (lane & 15)]);
+    float scale, iv;
+    pow2_scale_of(f32_bits(m), scale, iv);
+    if (wave == 0 && lane < 16) ainv[(u64) blockIdx.x * tok + 16 * T + lane] = iv * XPF_UNSCALE;
+    f32x4 rot[8];
+    xpf_rotate_tile([&](int ks) { return act[ks] * scale; }, hop, rot);
+    xpf_put_rows(arows + ((u64) blockIdx.x * (tok / 16) + T) * XPF_TILE_U16, wave, rot, lane);
+}
+
+// Launch 3: item blockIdx.x, 128-column blocks 4 blockIdx.y + w of hidden for wave w: the products of the item's operand rows
+// (copied from launch 2's into LDS, wave w its block w of every tile) over the ff / 128 input blocks and the output side:
+// eo[pair][hidden].  grid = (bound on the items, ceil(hidden / 512)), block 256, dynamic LDS 4 XPF_LDS_WORDS.
 template <int K>
 __device__ __forceinline__ void prefill_down_exl3_kernel(const u64* __restrict__ eaddr, const u64* __restrict__ sh_addr, const u32* __restrict__ offs,
-                                                         const u32* __restrict__ list, const u32* __restrict__ items, const float* __restrict__ gup,
-                                                         float* __restrict__ eo, u32 ne, u32 k, u32 npairs, u32 NP, u32 hidden, u32 ff, u32 zs) {
-    typedef Exl3Rows<K, 4> R;
+                                                         const u32* __restrict__ list, const u32* __restrict__ items, const u16* __restrict__ arows_g,
+                                                         const float* __restrict__ ainv, float* __restrict__ eo, u32 ne, u32 k, u32 npairs, u32 hidden, u32 ff) {
+    typedef Exl3Rows<K, XPF_D(K)> R;
+    constexpr u32 TOK = XPF_TOK(K);
     extern __shared__ __attribute__((aligned(16))) u32 dyn[];
     u16* arows = (u16*) dyn;
-    u32* rings = dyn + 4 * 8 * XPF_TOK * 8;
+    u32* rings = dyn + XPF_NT(K) * (XPF_TILE_U16 / 2);
     u32* s_pairs = rings + 4 * R::words;
-    u32* s_rows = s_pairs + XPF_TOK;
-    float* s_max = (float*) (s_rows + XPF_TOK);
-    float* s_pre = s_max + 4 * XPF_TOK;
+    u32* s_rows = s_pairs + TOK;
     const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
     const u32 kbs = ff / 128;                                  // at most 4
     u32 e;
-    const u32 nt = xpf_item(offs, list, items, blockIdx.x, ne, sh_addr != nullptr, k, npairs, s_pairs, s_rows, e);
+    const u32 nt = xpf_item(offs, list, items, blockIdx.x, ne, sh_addr != nullptr, k, npairs, TOK, s_pairs, s_rows, e);
     if (nt == 0) return;
-    const bool two = nt > 16;
+    const u32 ntiles = (nt + 15) / 16;
     const u8* down = (const u8*) (e < ne ? eaddr[2ull * ne + e] : sh_addr[2]);
-    __syncthreads();
-    u32 hop[2];
-    xpf_sign_tile(lane, hop);
-    f32x4 rot[2][8];
-    float mx[2][4];
-    if (wave < kbs) {
-        const u16* suh = (const u16*) down + wave * 128 + 4 * (lane >> 4);
-        typedef u16 u16x4 __attribute__((ext_vector_type(4)));
-        float sc[8][4];
-#pragma unroll
-        for (int ks = 0; ks < 8; ks++) {
-            const u16x4 s4 = *(const u16x4*) (suh + 16 * ks);
-#pragma unroll
-            for (int q = 0; q < 4; q++) sc[ks][q] = f16_to_f32(s4[q]);
-        }
-#pragma unroll
-        for (int T = 0; T < 2; T++) {
-            if (T == 1 && !two) break;
-            const u32 pair = s_pairs[16 * T + (lane & 15)];
-            const float* pg = gup + ((u64) pair * zs) * ff + wave * 128 + 4 * (lane >> 4);
-            const float* pu = gup + (((u64) NP + pair) * zs) * ff + wave * 128 + 4 * (lane >> 4);
-            f32x4 av[8];
-#pragma unroll
-            for (int ks = 0; ks < 8; ks++) {
-                f32x4 g = *(const f32x4*) (pg + 16 * ks), u = *(const f32x4*) (pu + 16 * ks);
-                for (u32 zz = 1; zz < zs; zz++) {
-                    g += *(const f32x4*) (pg + (u64) zz * ff + 16 * ks);
-                    u += *(const f32x4*) (pu + (u64) zz * ff + 16 * ks);
-                }
-#pragma unroll
-                for (int q = 0; q < 4; q++) av[ks][q] = (siluf_ref(g[q]) * u[q]) * sc[ks][q];
-            }
-            xpf_rotate_scaled(av, hop, rot[T], s_pre + wave * 16, lane);
-            xpf_token_max(rot[T], mx[T]);
-            if ((lane & 15) == 0) {
-#pragma unroll
-                for (int q = 0; q < 4; q++) s_max[wave * XPF_TOK + 16 * T + 4 * (lane >> 4) + q] = mx[T][q];
-            }
-        }
-    }
-    __syncthreads();
-    float inv[2][4];
-#pragma unroll
-    for (int T = 0; T < 2; T++)
-#pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const u32 t = 16 * T + 4 * (lane >> 4) + q;
-            float m = 0.0f;
-            for (u32 w = 0; w < kbs; w++) m = fmaxf(m, s_max[w * XPF_TOK + t]);
-            float scale, iv;
-            pow2_scale_of(f32_bits(m), scale, iv);
-            inv[T][q] = iv;
-            mx[T][q] = scale * 0.08838835f;
-        }
-    if (wave < kbs) {
-        xpf_put_a_rows(arows + wave * (8 * XPF_TOK * 16), 0, rot[0], mx[0], lane);
-        if (two) xpf_put_a_rows(arows + wave * (8 * XPF_TOK * 16), 1, rot[1], mx[1], lane);
-    }
-    __syncthreads();
     const u32 cb = 4 * blockIdx.y + wave;
-    if (cb >= hidden / 128) return;
+    const bool live = cb < hidden / 128;
+    // what undoes the powers of two of the lane's tokens (the only ordinary loads: consumed before the burst)
+    float iv[XPF_NT(K)];
+#pragma unroll
+    for (int T = 0; T < XPF_NT(K); T++) iv[T] = (u32) T < ntiles ? ainv[(u64) blockIdx.x * TOK + 16 * T + (lane & 15)] : 0.0f;
+#pragma unroll
+    for (int T = 0; T < XPF_NT(K); T++) asm volatile("" : "+v"(iv[T]));
     const u32 wb_lds = __builtin_amdgcn_readfirstlane(lds_offset(rings + wave * R::words));
+    if (wave < kbs) {
+        // block `wave` of every live tile: 8 tile rows of 512 bytes, 1 KiB a load
+        for (u32 T = 0; T < ntiles; T++) {
+            const u8* src = (const u8*) (arows_g + ((u64) blockIdx.x * XPF_NT(K) + T) * XPF_TILE_U16 + wave * 8 * 256);
+            const u32 dst = __builtin_amdgcn_readfirstlane(lds_offset(arows + T * XPF_TILE_U16 + wave * 8 * 256));
+#pragma unroll
+            for (int i = 0; i < 4; i++) lds_load<16>(src + i * 1024 + lane * 16, dst + i * 1024);
+        }
+    }
     const u64 pitch = (u64) (hidden / 16) * EXL3_TILE_WORDS(K, false);
-    const u32* row0 = (const u32*) (down + 2 * (u64) ff + 2 * (u64) hidden + 4) + (u64) cb * 8 * EXL3_TILE_WORDS(K, false);
-    exl3_rows_issue<K, 4>(row0, pitch, lane, wb_lds);
-    f32x4 acc[2][8];
-    xpf_wave_products<K>(row0, pitch, 8 * kbs, rings + wave * R::words, wb_lds, arows, two, lane, acc);
-    const u16* svh = (const u16*) (down + 2 * (u64) ff) + cb * 128 + (lane & 15);
-    float sv[8];
+    const u32* row0 = (const u32*) (down + 2 * (u64) ff + 2 * (u64) hidden + 4) + (u64) (live ? cb : 0) * 8 * EXL3_TILE_WORDS(K, false);
+    if (live) {
+        exl3_rows_issue<K, XPF_D(K)>(row0, pitch, lane, wb_lds);
+        wait_vm<R::loads>();                                  // this wave's operand rows have landed (its ring may still be on its way)
+    } else wait_vm<0>();
+    __syncthreads();                                          // every wave's operand rows, and the item's pairs
+    if (!live) return;
+    f32x4 acc[XPF_NT(K)][8];
+    xpf_wave_products<K>(row0, pitch, 8 * kbs, rings + wave * R::words, wb_lds, arows, ntiles, lane, acc);
+    typedef u16 u16x4 __attribute__((ext_vector_type(4)));
+    const u16* svh = (const u16*) (down + 2 * (u64) ff) + cb * 128;
+    f32x4 sv[8];
 #pragma unroll
-    for (int c = 0; c < 8; c++) sv[c] = f16_to_f32(svh[16 * c]) * 0.08838835f;
+    for (int c = 0; c < 8; c++) {
+        const u16x4 s4 = *(const u16x4*) (svh + xpf_out_col(c, lane));
 #pragma unroll
-    for (int T = 0; T < 2; T++) {
-        if (T == 1 && !two) break;
+        for (int q = 0; q < 4; q++) sv[c][q] = f16_to_f32(s4[q]) * 0.08838835f;
+    }
 #pragma unroll
-        for (int c = 0; c < 8; c++)
+    for (int T = 0; T < XPF_NT(K); T++) {
+        if ((u32) T >= ntiles) break;
 #pragma unroll
-            for (int q = 0; q < 4; q++) acc[T][c][q] *= inv[T][q];
-        xpf_output_side(acc[T], sv, lane);
+        for (int c = 0; c < 8; c++) acc[T][c] *= iv[T];
+        xpf_output_side(acc[T]);
+        const u32 t = 16 * T + (lane & 15);
+        if (t < nt) {
+            float* o = eo + (u64) s_pairs[t] * hidden + cb * 128;
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const u32 t = 16 * T + 4 * (lane >> 4) + q;
-            if (t < nt) {
-                float* o = eo + (u64) s_pairs[t] * hidden + cb * 128 + (lane & 15);
-#pragma unroll
-                for (int c = 0; c < 8; c++) o[16 * c] = acc[T][c][q];
-            }
+            for (int c = 0; c < 8; c++) *(f32x4*) (o + xpf_out_col(c, lane)) = acc[T][c] * sv[c];
         }
     }
 }
@@ -2219,9 +2259,9 @@ __device__ __forceinline__ void prefill_down_exl3_kernel(const u64* __restrict__
         prefill_gate_up_exl3_kernel<K>(eaddr, sh_addr, offs, list, items, x, gup, ne, k, npairs, NP, hidden, ff);                        \
     }                                                                                                                                    \
     extern "C" __global__ void __launch_bounds__(256, 2) prefill_down_exl3_##K(const u64* eaddr, const u64* sh_addr, const u32* offs, const u32* list, \
-                                                                                const u32* items, const float* gup, float* eo, u32 ne, u32 k, u32 npairs, \
-                                                                                u32 NP, u32 hidden, u32 ff, u32 zs) {                    \
-        prefill_down_exl3_kernel<K>(eaddr, sh_addr, offs, list, items, gup, eo, ne, k, npairs, NP, hidden, ff, zs);                      \
+                                                                                const u32* items, const u16* arows, const float* ainv, float* eo, u32 ne, \
+                                                                                u32 k, u32 npairs, u32 hidden, u32 ff) {                 \
+        prefill_down_exl3_kernel<K>(eaddr, sh_addr, offs, list, items, arows, ainv, eo, ne, k, npairs, hidden, ff);                      \
     }
 EXL3_PREFILL_ENTRIES(1)
 EXL3_PREFILL_ENTRIES(2)
