@@ -153,9 +153,10 @@ void sz_session_free(sz_session*);
  * one type; `shared` (0: none) is the shared expert in the same layout and of type shared_type. */
 int32_t sz_session_set_layer(sz_session*, uint32_t layer, int32_t expert_type, uint64_t experts, uint64_t stride, int32_t shared_type,
                              uint64_t shared);
-/* output.weight, vocab x hidden: Q8_0 or IQ3_S rows, or an EXL3 blob at a whole bit rate (in = hidden, out = vocab, both
- * multiples of 128; the head of an EXL3 checkpoint, session.rs:7179-7187).  The fused arg-max (sz_head_argmax,
- * sz_verify_round) exists for Q8_0 and EXL3; logits and the top 64 for all three. */
+/* output.weight, vocab x hidden: Q8_0, IQ3_S, F32, F16 or BF16 rows, or an EXL3 blob at a whole bit rate (in = hidden, out =
+ * vocab, both multiples of 128; the head of an EXL3 checkpoint, session.rs:7179-7187).  The arg-max (sz_head_argmax,
+ * sz_verify_round) is fused into the product for Q8_0 and EXL3; the other types go through their logits, kept in a buffer
+ * this call allocates (max_rows x vocab floats), as the reference's mv_cols + topk_rows_at do (session.rs:7034-7052). */
 int32_t sz_session_set_head(sz_session*, int32_t ggml_type, uint64_t w);
 /* LDS a workgroup of the EXL3 head's kernel takes for m rows (0 for another type): the head entry points refuse a call
  * whose need is above a compute unit's 160 KiB (hidden 4096 takes all 8 rows at any rate, hidden 8192 up to 4), and

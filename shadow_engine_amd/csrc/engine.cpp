@@ -622,7 +622,9 @@ int head_check(sz_session* s, uint32_t m, uint64_t u, const char* who) {
     return 0;
 }
 
-bool head_argmax_supported(const sz_session* s) { return s->head_type == SZ_TYPE_Q8_0 || head_is_exl3(s); }
+// Q8_0 and EXL3 heads have the arg-max fused into the product; every other type goes through its logits (set_head keeps the
+// buffer for them).
+bool head_argmax_fused(const sz_session* s) { return s->head_type == SZ_TYPE_Q8_0 || head_is_exl3(s); }
 
 // An EXL3 head (kernels/exl3.cu:349-461, 610-625 of the reference: rotate the rows once, then one pass over the matrix for all
 // m <= 8 rows): the arg-max ids (0: not wanted) and / or the logits (0: not written).
@@ -686,9 +688,20 @@ int head_proxy_sparse(sz_session* s, uint32_t m, uint64_t u, uint32_t need_k, ui
     return 0;
 }
 
+int head_logits(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uint64_t stream);
+
 int head_argmax(sz_session* s, uint32_t m, uint64_t u, uint64_t ids, uint64_t stream) {
     if (head_check(s, m, u, "sz_head_argmax")) return 1;
-    if (!head_argmax_supported(s)) return fail("sz_head_argmax: the head's type has no fused arg-max kernel (Q8_0 or EXL3)");
+    if (!head_argmax_fused(s)) {
+        // mv_cols + topk_rows_at (session.rs:7034-7052): the logits, the largest of every slice of 4096, the largest of those
+        const sz_session_config& c = s->cfg;
+        const uint32_t nparts = (c.vocab + 4095) / 4096;
+        if (head_logits(s, m, u, s->logits.ptr, stream)) return 1;
+        const sz_arg a[] = {P(s->logits.ptr), U32(c.vocab), U32(c.vocab), P(s->head_part.ptr), U32(8)};
+        if (launch("argmax_slices", nparts, m, 1, 256, 0, stream, a)) return 1;
+        const sz_arg b[] = {P(s->head_part.ptr), U32(nparts), U32(8), P(ids), P(0)};
+        return launch("argmax_merge_parts", m, 1, 1, 256, 0, stream, b);
+    }
     if (head_is_exl3(s)) return head_exl3(s, m, u, 0, ids, stream);
     if (head_mfma_ok(s)) return head_argmax_mfma(s, m, u, 0, ids, stream);
     for (uint32_t j0 = 0; j0 < m; j0 += 4) {
@@ -836,7 +849,11 @@ int32_t sz_session_set_head(sz_session* s, int32_t ty, uint64_t w) {
     clear_error();
     if (!s) return fail("sz_session_set_head: null session");
     const bool exl3 = ty >= 1021 && ty <= 1028;
-    if (ty != SZ_TYPE_Q8_0 && ty != SZ_TYPE_IQ3_S && !exl3) return fail("sz_session_set_head: the head must be Q8_0, IQ3_S or EXL3 at a whole bit rate");
+    const bool plain = ty == SZ_TYPE_F32 || ty == SZ_TYPE_F16 || ty == SZ_TYPE_BF16;
+    if (ty != SZ_TYPE_Q8_0 && ty != SZ_TYPE_IQ3_S && !plain && !exl3)
+        return fail("sz_session_set_head: the head must be Q8_0, IQ3_S, F32, F16, BF16 or EXL3 at a whole bit rate");
+    // a type without a fused arg-max keeps its logits: allocated here, never during a call (a call may be under capture)
+    if (ty != SZ_TYPE_Q8_0 && !exl3 && s->logits.need((uint64_t) s->cfg.max_rows * s->cfg.vocab * 4)) return 1;
     if (w & 15) return fail("sz_session_set_head: the head must be 16-byte aligned");
     if (exl3) {
         const sz_session_config& c = s->cfg;
@@ -1020,7 +1037,6 @@ int32_t sz_verify_round(sz_session* s, uint32_t m, uint64_t u, uint64_t rl, uint
     const sz_session_config& c = s->cfg;
     // everything that can be refused is refused before a capture begins
     if (head_check(s, m, head_u, "sz_verify_round")) return 1;
-    if (!head_argmax_supported(s)) return fail("sz_verify_round: the head's type has no fused arg-max kernel (Q8_0 or EXL3)");
     for (uint32_t l = 0; l < c.n_layers; l++)
         if (!s->layers[l].set) return fail("sz_verify_round: layer " + std::to_string(l) + " has no experts set");
     const SzGraphKey key{{m, u, rl, sgl, y, head_u, drafts, out, stream, 0}};

@@ -1313,6 +1313,40 @@ extern "C" __global__ void __launch_bounds__(512) head_q8_0_argmax_mfma_w8(const
     head_mfma_body<8>(w, x, xs, logits, ls, part, rows, cols, m);
 }
 
+// part[(p * ts + j) * 2], + 1 = the largest of slice p (4096 values) of row j of logits (rows ls apart, n values a row) and its
+// index, ties to the lower index: the first step of the arg-max for a head whose product kernel has none fused in (any type
+// matvec_cols takes; the reference's mv_cols + topk_rows_at, session.rs:7034-7052).  grid = (ceil(n / 4096), m), block 256.
+extern "C" __global__ void __launch_bounds__(256) argmax_slices(const float* logits, u32 ls, u32 n, u32* part, u32 ts) {
+    __shared__ float sv[256];
+    __shared__ u32 si[256];
+    const u32 p = blockIdx.x, j = blockIdx.y, tid = threadIdx.x;
+    const float* row = logits + (u64) j * ls;
+    float bv = -__builtin_inff();
+    u32 bi = 0xffffffffu;
+#pragma unroll 4
+    for (u32 q = 0; q < 16; q++) {
+        const u32 i = p * 4096 + q * 256 + tid;
+        if (i < n) argmax_merge(bv, bi, row[i], i);
+    }
+    sv[tid] = bv;
+    si[tid] = bi;
+    __syncthreads();
+    for (u32 s = 128; s > 0; s >>= 1) {
+        if (tid < s) {
+            float v = sv[tid];
+            u32 i = si[tid];
+            argmax_merge(v, i, sv[tid + s], si[tid + s]);
+            sv[tid] = v;
+            si[tid] = i;
+        }
+        __syncthreads();
+    }
+    if (tid == 0) {
+        part[((u64) p * ts + j) * 2] = f32_bits(sv[0]);
+        part[((u64) p * ts + j) * 2 + 1] = si[0];
+    }
+}
+
 // ids[j] = index of the largest of row j's `nparts` partial maxima part[(p * ts + j) * 2] (ties to the lower index).
 // grid = m, block 256.
 extern "C" __global__ void __launch_bounds__(256) argmax_merge_parts(const u32* part, u32 nparts, u32 ts, u32* ids, float* vals) {

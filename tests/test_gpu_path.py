@@ -877,12 +877,58 @@ def test_verify_round_with_an_exl3_head(gpu):
         stream.synchronize()
         o = out.cpu().numpy().view(np.uint32)
         assert np.array_equal(o[2:2 + m], want_ids) and o[0] == 3 and o[1] == want_ids[2]
-    # a head without a fused arg-max is refused before anything is captured
+    # a head whose product has no arg-max fused in goes through its logits (the reference's mv_cols + topk_rows_at,
+    # session.rs:7034-7052): the same round, captured anew for the new head
     wq = synth.iq3_s_matrix(rng, vocab, hidden)
     dq = dev(gpu, wq)
     s.set_head(sz.IQ3_S, dq.data_ptr())
-    with pytest.raises(sz.SzError, match="no fused arg-max"):
-        s.verify_round(m, du.data_ptr(), drl.data_ptr(), dsgl.data_ptr(), y.data_ptr(), dhu.data_ptr(), dd.data_ptr(), out.data_ptr(), stream.handle)
+    want = [O.matvec(sz.IQ3_S, hidden, vocab, wq, hu[j]) for j in range(m)]
+    assert all(clear_gap(w) for w in want)
+    want_ids = np.array([O.argmax(w) for w in want], np.uint32)
+    drafts = want_ids[:m - 1].copy()
+    drafts[1] = (drafts[1] + 1) % vocab                      # one of the three drafts is accepted
+    dd2 = dev(gpu, drafts.astype(np.int32))
+    for replay in range(3):
+        out.zero_()
+        gpu.cuda.synchronize()
+        s.verify_round(m, du.data_ptr(), drl.data_ptr(), dsgl.data_ptr(), y.data_ptr(), dhu.data_ptr(), dd2.data_ptr(), out.data_ptr(), stream.handle)
+        stream.synchronize()
+        o = out.cpu().numpy().view(np.uint32)
+        assert np.array_equal(o[2:2 + m], want_ids) and o[0] == 2 and o[1] == want_ids[1]
+
+
+@pytest.mark.parametrize("ty", ["iq3_s", "f32", "f16", "bf16"])
+def test_head_argmax_of_a_type_without_a_fused_kernel(gpu, ty):
+    """sz_head_argmax for heads that are neither Q8_0 nor EXL3 (session.rs:7034-7052 takes any type): the oracle's arg-max of
+    the oracle's logits on rows with a clear gap, the lowest id on exact ties (equal rows of the matrix in different slices of
+    4096), a vocabulary that is no multiple of the slice, 1 to 8 rows."""
+    t = {"iq3_s": sz.IQ3_S, "f32": sz.F32, "f16": sz.F16, "bf16": sz.BF16}[ty]
+    rng = np.random.default_rng(77 + t)
+    vocab, hidden = 9001, 512
+    if t == sz.IQ3_S:
+        w = synth.iq3_s_matrix(rng, vocab, hidden).reshape(vocab, -1)
+    else:
+        w = dense_matrix(rng, t, vocab, hidden).reshape(vocab, -1)
+    u = rng.normal(size=(8, hidden)).astype(np.float32)
+    base = O.matvec(t, hidden, vocab, w.reshape(-1), u[0])
+    best = int(np.argmax(base))
+    twins = [i for i in (17, 4100, 9000) if i != best]
+    for i in twins:
+        w[i] = w[best]                                       # row 0's largest logit now occurs at several ids
+    dw, du = dev(gpu, w.reshape(-1)), dev(gpu, u)
+    s = sz.Session(hidden, 512, 8, 2, 0, vocab, 8)
+    s.set_head(t, dw.data_ptr())
+    want = [O.matvec(t, hidden, vocab, w.reshape(-1), u[j]) for j in range(8)]
+    for m in (1, 3, 8):
+        ids = gpu.zeros(8, dtype=gpu.int32, device="cuda")
+        s.head_argmax(m, du.data_ptr(), ids.data_ptr())
+        gpu.cuda.synchronize()
+        got = ids.cpu().numpy().view(np.uint32)
+        assert got[0] == min([best] + twins)
+        for j in range(1, m):
+            if clear_gap(want[j]):
+                assert got[j] == O.argmax(want[j]), (m, j)
+        assert not got[m:].any()
 
 
 def test_head_argmax_prefers_the_lowest_id_on_exact_ties(gpu):
