@@ -73,9 +73,10 @@ class Workload:
         pass
 
 
-def exl3_round(torch, sz, synth, synth_device, stream, L, rates, tag):
+def exl3_round(torch, sz, synth, synth_device, stream, L, rates, tag, mode=0):
     w = Workload()
     sess = sz.Session(HIDDEN, FF, NE, TOPK, L, VOCAB, 8)
+    sess.set_expert_mode(mode)   # 0: the exact kernels (the default); 1, 2: the matrix-core launches
     layers = []
     for l, kb in enumerate(rates):
         buf, stride = synth_device.exl3_layer(torch, 1000 + l, HIDDEN, FF, NE, kb)
@@ -133,11 +134,15 @@ def exl3_round(torch, sz, synth, synth_device, stream, L, rates, tag):
     w.step, w.check, w.set_eager = step, check, (lambda eager: sess.set_graph(not eager))
     w.step_bytes = moe_bytes + head_bytes + act_bytes
     w.counters_key = "config5" if (L == 48 and tag == "config 5" and ROWS == 4) else ("config3" if (tag == "config 3" and ROWS == 4) else None)
+    if mode:
+        w.counters_key = "config5_mode%d" % mode if w.counters_key == "config5" else None
     w.cold_variant = tag == "config 3"
     w.dtype = "f32 accumulate over EXL3 f16 codebook weights / Q8_0 int8"
     w.describe = {"workload": "%s: verify round, %d MoE layer%s (hidden 2048, 512 experts + shared, top-10, EXL3 K in %s), %d-token batch, "
                               "Q8_0 lm_head 151936x2048, arg-max, greedy acceptance of %d drafts" % (tag, L, "s" if L > 1 else "", sorted(set(rates)), ROWS, ROWS - 1),
                   "layers": L, "rows": ROWS, "resident_GB": round(sum(b.numel() for b, _ in layers) / 1e9 + head.numel() / 1e9, 2)}
+    if mode:
+        w.describe["expert_mode"] = {1: "matrix cores, the codebook's f16 values", 2: "matrix cores, the linearised codebook"}[mode]
     w.extra = {"accepted_drafts": wrong}
     w.cpu = ("exl3_token", (layers[0], rates[0], rl_h[0], u[0].cpu().numpy(), sgl[0].cpu().numpy()))
     w.keep = (sess, layers, head, u, rl, sgl, hu, y, out, drafts)
@@ -606,9 +611,9 @@ def cpu_baseline(kind, args, budget_s=8.0):
 
 def build_workload(name, torch, sz, synth, synth_device, stream, args):
     if name == "config5":
-        return exl3_round(torch, sz, synth, synth_device, stream, args.layers, synth_device.layer_rates(2026, args.layers), "config 5")
+        return exl3_round(torch, sz, synth, synth_device, stream, args.layers, synth_device.layer_rates(2026, args.layers), "config 5", args.expert_mode)
     if name == "config3":
-        return exl3_round(torch, sz, synth, synth_device, stream, 1, [3], "config 3")
+        return exl3_round(torch, sz, synth, synth_device, stream, 1, [3], "config 3", args.expert_mode)
     if name == "config1":
         return q8_matvec(torch, sz, synth, synth_device, stream)
     if name == "config2":
@@ -636,6 +641,8 @@ def main():
     ap.add_argument("--rows", type=int, default=4, help="rows of the verify batch (config3, config5, exl3head; the configurations name 4; 1..8)")
     ap.add_argument("--tokens", type=int, default=512, help="tokens of the prefill chunk (config4 only; the configuration names 512)")
     ap.add_argument("--bits", type=int, default=0, help="bits a weight of the EXL3 head (exl3head, exl3top: 4 unless given) or of the chunk's experts (exl3prefill: 3)")
+    ap.add_argument("--expert-mode", type=int, default=0, choices=[0, 1, 2],
+                    help="config3, config5: 0 the exact EXL3 expert kernels (the library's default), 1 the matrix-core launches with the codebook's f16 values, 2 with the linearised codebook")
     ap.add_argument("--screen", type=int, default=0, help="exl3top: blocks a row of the inexact 2-bit screen (0: the exact hand-off)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true", help="default workload only: do not time configurations 1-4 after it")
