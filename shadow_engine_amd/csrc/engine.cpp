@@ -320,6 +320,8 @@ struct sz_session {
     uint64_t head_w = 0;
     // batch buffers (session.rs `bb`): the plan, the expert products, the split-k partials, the head's scratch
     DevBuf plan, eg, act, eo, part, dn, head_part, logits, topv, topi, ids;
+    DevBuf plans;                 // a plan a layer for the rounds that route every layer up front (sz_verify_round)
+    uint32_t plan_stride = 0;
     DevBuf head_xa, head_inv;   // an EXL3 head's rotated inputs as f16 high and low parts (16 rows of 128 a 128-block), and the tokens' scales
     DevBuf rl, sgl;   // the router's outputs for a batch: f32[max_rows][n_expert], f32[max_rows]
     // the optional 2-bit screen of an EXL3 head (HeadProxy of session.rs:428-441): k_blk = 0 is off
@@ -389,6 +391,10 @@ struct PendingSum {
     bool active = false;
     uint64_t plan = 0, sgl = 0, y = 0;
     bool shared = false;
+    // the round's routing launch (verify_route_layers) has filled a plan a layer, `plan_stride` apart from `plans` on: the
+    // exact EXL3 launches of those layers get no logits and read their plan instead of redoing the selection
+    uint64_t plans = 0;
+    uint32_t plan_stride = 0;
 };
 
 int launch_pending_sum(sz_session* s, PendingSum& ps, uint32_t m, uint64_t stream) {
@@ -412,8 +418,11 @@ int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, ui
     const bool shared = L.shared != 0;
     if (shared && L.shared_type != L.type) return fail("the shared expert must have the routed experts' type (layer " + std::to_string(l) + ")");
     const PlanLayout p = plan_layout(m, c.top_k);
-    // a layer whose sum may ride the next launch takes the plan buffer the pending sum is not reading
-    const uint64_t plan = (ride && ride->active && ride->plan == s->plan.ptr) ? s->plan2.ptr : s->plan.ptr;
+    // a layer whose sum may ride the next launch takes the plan buffer the pending sum is not reading; a layer routed by the
+    // round's routing launch has a plan of its own
+    const bool routed = ride && ride->plans && f.exl3 && s->expert_mode == 0;
+    const uint64_t plan = routed ? ride->plans + (uint64_t) l * ride->plan_stride
+                                 : (ride && ride->active && ride->plan == s->plan.ptr) ? s->plan2.ptr : s->plan.ptr;
     s->last_plan = plan;
     const uint64_t addr = plan + p.a0, rec = plan + p.r0, wts = plan + p.w_off, cnt = plan + p.counts_off;
     const uint64_t addr_d = addr + 2ull * p.GT * 8, rec_d = rec + 2ull * p.GT * 17 * 4;
@@ -429,7 +438,11 @@ int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, ui
         if (ride) ride->active = false;
         s->last_fused = true;
         if (ride && zs_d == 1) {
-            *ride = PendingSum{true, plan, sgl, y, shared};
+            ride->active = true;
+            ride->plan = plan;
+            ride->sgl = sgl;
+            ride->y = y;
+            ride->shared = shared;
             return 0;
         }
         const sz_arg a[] = {P(s->dn.ptr), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(plan), P(sgl), P(y),
@@ -472,12 +485,12 @@ int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, ui
         const std::string k1 = "verify_gate_up_" + tag, k2 = "verify_down_" + tag;
         {
             const uint32_t gx = c.ff / 128, extra = (carry_groups + gx * zs_gu - 1) / (gx * zs_gu);   // rows of the grid for a riding sum
-            const sz_arg a[] = {P(rl), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(u), P(plan), P(s->part.ptr),
+            const sz_arg a[] = {P(routed ? 0 : rl), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(u), P(plan), P(s->part.ptr),
                                 U32(c.n_expert), U32(c.top_k), U32(m), U32(c.hidden), U32(c.ff), P(s->dn.ptr), P(c_plan), P(c_sgl), P(c_y), U32(c_mode)};
             if (launch(k1.c_str(), gx, 2 * S + extra, zs_gu, 256, 0, stream, a)) return 1;   // 4 waves of one 128-block each: EXL3_GU_WAVES, EXL3_VERIFY_NB
         }
         {
-            const sz_arg a[] = {P(rl), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(plan), P(s->part.ptr), P(s->dn.ptr),
+            const sz_arg a[] = {P(routed ? 0 : rl), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(plan), P(s->part.ptr), P(s->dn.ptr),
                                 U32(c.n_expert), U32(c.top_k), U32(m), U32(c.hidden), U32(c.ff), U32(zs_gu)};
             if (launch(k2.c_str(), c.hidden / 128, S, zs_d, 256, 0, stream, a)) return 1;
         }
@@ -744,6 +757,8 @@ sz_session* sz_session_new(const sz_session_config* cfg) {
                s->eo.need((uint64_t) p.R * c.hidden * 4) || s->part.need(part) || s->ids.need(64) ||
                s->dn.need((uint64_t) p.GT * ks_d * 4 * c.hidden * 4);
     if (c.vocab) bad = bad || s->head_part.need(nparts * 4 * 2 * 4);
+    s->plan_stride = (uint32_t) ((2ull * c.max_rows * c.top_k * 4 + c.max_rows * 4 + 255) & ~255ull);
+    if (c.n_layers) bad = bad || s->plans.need((uint64_t) c.n_layers * s->plan_stride);
     if (bad) {
         delete s;
         return nullptr;
@@ -1046,6 +1061,16 @@ int32_t sz_verify_round(sz_session* s, uint32_t m, uint64_t u, uint64_t rl, uint
         auto record = [&]() -> int {
             // an EXL3 layer's rank-order sum rides the first launch of the layer after it; the last layer's gets its own launch
             PendingSum ps;
+            bool any_exl3 = false;
+            for (uint32_t l = 0; l < c.n_layers; l++) any_exl3 = any_exl3 || (s->layers[l].type >= 1021 && s->layers[l].type <= 1033);
+            static const bool route_in_launch = std::getenv("SHADOWZERO_ROUTE_IN_LAUNCH") != nullptr;   // the form without the routing launch, for comparisons
+            if (any_exl3 && s->expert_mode == 0 && !route_in_launch) {
+                // every layer's router logits are inputs of the round: all of them are routed by one launch before the first layer
+                const sz_arg a[] = {P(rl), P(s->plans.ptr), U32(s->plan_stride), U32(c.n_expert), U32(c.top_k), U32(m), U32(c.n_layers)};
+                if (launch("verify_route_layers", (c.n_layers * m + 3) / 4, 1, 1, 256, 0, stream, a)) return 1;
+                ps.plans = s->plans.ptr;
+                ps.plan_stride = s->plan_stride;
+            }
             for (uint32_t l = 0; l < c.n_layers; l++) {
                 const uint64_t off = (uint64_t) l * m;
                 if (moe_layer(s, l, m, u + off * c.hidden * 4, rl + off * c.n_expert * 4, sgl + off * 4, y + off * c.hidden * 4, stream, &ps)) return 1;

@@ -499,6 +499,32 @@ __device__ __forceinline__ void exl3_combine_finished(const float* __restrict__ 
     y[(u64) j * hidden + col] = a;
 }
 
+// The routing of a whole round in one launch, for a caller that has every layer's router logits before the first layer runs
+// (sz_verify_round): wave (l, j) leaves token j's chosen experts, weights and count in layer l's plan, plans + l *
+// plan_stride, in the layout above; launches 1 and 2 of those layers are then given no logits and read the plan instead of
+// redoing the selection in every workgroup.  Same functions as the launches use, so the same bits.
+// logits[l][m][ne]; grid = ceil(L m / 4), block 256; ne <= 512, k <= 16.
+extern "C" __global__ void __launch_bounds__(256) verify_route_layers(const float* logits, u8* plans, u32 plan_stride, u32 ne, u32 k, u32 m, u32 L) {
+    __shared__ double exs[4][512];
+    __shared__ u32 tops[4][16];
+    const u32 lane = threadIdx.x & 63, w = threadIdx.x >> 6;
+    const u32 i = blockIdx.x * 4 + w;
+    if (i >= L * m) return;
+    const u32 l = i / m, j = i - l * m, G = m * k;
+    const float* lg = logits + (u64) i * ne;
+    u8* pbuf = plans + (u64) l * plan_stride;
+    route_ids(lg, ne, k, lane, exs[w], tops[w]);
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    u32 kk;
+    const float wt = route_weights(lg, ne, k, lane, tops[w], &kk);
+    if (lane < k) {
+        ((u32*) pbuf)[j * k + lane] = tops[w][lane];
+        ((float*) (pbuf + G * 4))[j * k + lane] = wt;
+    }
+    if (lane == 0) ((u32*) (pbuf + 2 * G * 4))[j] = kk;
+}
+
 // Launch 1's workgroup: EXL3_GU_WAVES waves, each takes EXL3_VERIFY_NB consecutive 128-blocks of the input through a ring
 // of EXL3_GU_DEPTH rows (grid z = ceil(hidden / 128 / (waves * blocks))).  One block a wave with a 4-row ring puts twice as
 // many waves on a SIMD as two blocks a wave with an 8-row ring, for the same LDS: the waves spend most of their life
@@ -554,7 +580,12 @@ __device__ __forceinline__ void verify_gate_up_kernel(const float* __restrict__ 
     }
     u32* tidx = (u32*) pbuf;
     const u8* bp;
-    if (pair < G) {
+    if (pair < G && logits == nullptr) {
+        // the round's routing launch has left every layer's chosen experts in its plan (verify_route_layers): one load
+        const u32 e = tidx[pair];
+        if (e == 0xffffffffu) return;
+        bp = (const u8*) (ebase + e * estride + (u64) sel * part);
+    } else if (pair < G) {
         const u32 t = pair % k;
         if (wave == (blockIdx.x + blockIdx.y + blockIdx.z) % WA) {   // not always the same wave: the prologues of co-resident workgroups spread over the SIMDs
             // the selection is a chain of dependent steps that the whole workgroup waits for: it goes ahead of the decoding
@@ -629,7 +660,7 @@ __device__ __forceinline__ void verify_down_kernel(const float* __restrict__ log
     const u32 G = m * k, S = G + m;
     const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // the wave index as a scalar: the index arithmetic on it is the scalar unit's
     const u32 pair = blockIdx.y;
-    if (pair < G && pair % k == 0 && blockIdx.x == 0 && blockIdx.z == 0 && wave == 3) {
+    if (logits != nullptr && pair < G && pair % k == 0 && blockIdx.x == 0 && blockIdx.z == 0 && wave == 3) {
         // one wave a token: the routing weights and the count, for launch 3 (nothing in this launch reads them)
         const u32 j = pair / k;
         u32 kk;
