@@ -574,8 +574,8 @@ __device__ __forceinline__ void verify_gate_up_kernel(const float* __restrict__ 
         v[b][0] = v[b][1] = 0.0f;
         if ((u32) b < nb) {
             const float* xj = u + (u64) j * hidden + (kb0 + b) * 128;
-            v[b][0] = xj[lane];
-            v[b][1] = xj[lane + 64];
+            v[b][0] = load_f32_uncounted(xj + lane);      // waited for together with the input scales, behind which the trellis rows are already on their way
+            v[b][1] = load_f32_uncounted(xj + lane + 64);
         }
     }
     u32* tidx = (u32*) pbuf;
@@ -605,8 +605,6 @@ __device__ __forceinline__ void verify_gate_up_kernel(const float* __restrict__ 
     }
     float* xw = xw_all[wave];
     if (nb) {
-#pragma unroll
-        for (int b = 0; b < NB; b++) asm volatile("" : "+v"(v[b][0]), "+v"(v[b][1]));   // the row's values are here: no ordinary load is in flight from now on
         const u32 sc_lds = __builtin_amdgcn_readfirstlane(lds_offset(sc_all[wave]));
         const u32 wb_lds = __builtin_amdgcn_readfirstlane(lds_offset(wb_all[wave]));
         for (u32 b = 0; b < nb; b++) lds_load<4>(bp + (kb0 + b) * 256 + lane * 4, sc_lds + b * 256);
@@ -614,7 +612,12 @@ __device__ __forceinline__ void verify_gate_up_kernel(const float* __restrict__ 
         const u32* row0 = (const u32*) (bp + 2 * (u64) hidden + 2 * (u64) ff + 4) + ((u64) kb0 * 8 * (ff / 16) + blockIdx.x * 8) * EXL3_TILE_WORDS(K, H);
         const u64 pitch = (u64) (ff / 16) * EXL3_TILE_WORDS(K, H);
         exl3_rows_issue<K, D, H>(row0, pitch, lane, wb_lds);
-        wait_vm<Exl3Rows<K, D, H>::loads>();
+        wait_vm<Exl3Rows<K, D, H>::loads>();   // everything requested before the rows: the token's values, the scales
+#pragma unroll
+        for (int b = 0; b < NB; b++) {
+            load_landed(v[b][0]);
+            load_landed(v[b][1]);
+        }
         const u16* sc = (const u16*) sc_all[wave];
 #pragma unroll
         for (int b = 0; b < NB; b++) {
@@ -672,50 +675,35 @@ __device__ __forceinline__ void verify_down_kernel(const float* __restrict__ log
     const u32 kbs = ff / 128;
     // launch 1's partial sums of the wave's block of gate and up only depend on the pair: requested before its expert is known
     float g0 = 0.0f, g1 = 0.0f, u0 = 0.0f, u1 = 0.0f;
+    float pv[4][4];
     u32 e = 0;
     if (pair < G) e = ((const u32*) pbuf)[pair];
     if (kb < kbs) {
-        // the first four partials' loads all go out before any is waited for (a loop would take them a round trip at a time)
-        float pv[4][4];
+        // the first four partials' loads all go out before any is waited for (a loop would take them a round trip at a time),
+        // and without the compiler's count: the wave's rows are requested as soon as its expert is known, behind these loads
+        // and without waiting for them, and the sums are taken once exactly these have landed
 #pragma unroll
         for (int z = 0; z < 4; z++) {
             const u32 zz = min((u32) z, zs - 1);
             const float* pg = gup + ((u64) pair * zs + zz) * ff + kb * 128;
             const float* pu = gup + ((u64) (S + pair) * zs + zz) * ff + kb * 128;
-            pv[z][0] = pg[lane];
-            pv[z][1] = pg[lane + 64];
-            pv[z][2] = pu[lane];
-            pv[z][3] = pu[lane + 64];
-        }
-#pragma unroll
-        for (int z = 0; z < 4; z++) {
-            if ((u32) z < zs) {
-                g0 += pv[z][0];
-                g1 += pv[z][1];
-                u0 += pv[z][2];
-                u1 += pv[z][3];
-            }
-        }
-        for (u32 z = 4; z < zs; z++) {
-            const float* pg = gup + ((u64) pair * zs + z) * ff + kb * 128;
-            const float* pu = gup + ((u64) (S + pair) * zs + z) * ff + kb * 128;
-            g0 += pg[lane];
-            g1 += pg[lane + 64];
-            u0 += pu[lane];
-            u1 += pu[lane + 64];
+            pv[z][0] = load_f32_uncounted(pg + lane);
+            pv[z][1] = load_f32_uncounted(pg + lane + 64);
+            pv[z][2] = load_f32_uncounted(pu + lane);
+            pv[z][3] = load_f32_uncounted(pu + lane + 64);
         }
     }
     if (pair < G ? e == 0xffffffffu : shbase == 0) return;
     const u8* bp = (const u8*) (pair < G ? ebase + e * estride : shbase);
     float* xw = xw_all[wave];
-    float sv0 = 0.0f, sv1 = 0.0f;   // wave 0 of a launch without a split over the inputs: down's output scales of the block
+    u32 svb0 = 0, svb1 = 0;   // wave 0 of a launch without a split over the inputs: down's output scales of the block (needed at the end)
     if (gridDim.z == 1 && wave == 0) {
         const u16* svh = (const u16*) (bp + 2 * (u64) part + 2 * (u64) ff) + blockIdx.x * 128;
-        sv0 = f16_to_f32(svh[lane]);
-        sv1 = f16_to_f32(svh[lane + 64]);
+        svb0 = load_u16_uncounted(svh + lane);
+        svb1 = load_u16_uncounted(svh + lane + 64);
     }
     if (kb < kbs) {
-        asm volatile("" : "+v"(g0), "+v"(g1), "+v"(u0), "+v"(u1), "+v"(sv0), "+v"(sv1));   // no ordinary load is in flight from now on
+        // no load the compiler counts is in flight here: what is, is counted by hand
         const u32 sc_lds = __builtin_amdgcn_readfirstlane(lds_offset(sc_all[wave]));
         const u32 wb_lds = __builtin_amdgcn_readfirstlane(lds_offset(wb_all[wave]));
         const u8* down = bp + 2 * (u64) part;
@@ -723,6 +711,26 @@ __device__ __forceinline__ void verify_down_kernel(const float* __restrict__ log
         const u32* row0 = (const u32*) (down + 2 * (u64) ff + 2 * (u64) hidden + 4) + ((u64) kb * 8 * (hidden / 16) + blockIdx.x * 8) * EXL3_TILE_WORDS(K, H);
         const u64 pitch = (u64) (hidden / 16) * EXL3_TILE_WORDS(K, H);
         exl3_rows_issue<K, 8, H>(row0, pitch, lane, wb_lds);
+        wait_vm<Exl3Rows<K, 8, H>::loads + 1>();   // the partial sums, requested before the burst, have landed
+#pragma unroll
+        for (int z = 0; z < 4; z++) {
+#pragma unroll
+            for (int c = 0; c < 4; c++) load_landed(pv[z][c]);
+            if ((u32) z < zs) {
+                g0 += pv[z][0];
+                g1 += pv[z][1];
+                u0 += pv[z][2];
+                u1 += pv[z][3];
+            }
+        }
+        for (u32 z = 4; z < zs; z++) {   // (hidden above 2048: these wait for the burst too)
+            const float* pg = gup + ((u64) pair * zs + z) * ff + kb * 128;
+            const float* pu = gup + ((u64) (S + pair) * zs + z) * ff + kb * 128;
+            g0 += pg[lane];
+            g1 += pg[lane + 64];
+            u0 += pu[lane];
+            u1 += pu[lane + 64];
+        }
         // the wave's 128-block of act = silu(gate) * up (launch 1 left gate and up finished but for the sum over its
         // partials), rotated into the down projection's basis, into its strip
         wait_vm<Exl3Rows<K, 8, H>::loads>();
@@ -742,6 +750,10 @@ __device__ __forceinline__ void verify_down_kernel(const float* __restrict__ log
         // the workgroup holds the whole sum over the inputs: it finishes its block here (output-side transform, scales), and
         // launch 3 only weights and adds
         if (wave == 0) {
+            wait_vm<0>();
+            load_landed(svb0);
+            load_landed(svb1);
+            const float sv0 = f16_to_f32((u16) svb0), sv1 = f16_to_f32((u16) svb1);
             float a0 = xw_all[0][lane], a1 = xw_all[0][lane + 64];
             for (u32 w = 1; w < nw; w++) {
                 a0 += xw_all[w][lane];

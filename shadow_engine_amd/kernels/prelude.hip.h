@@ -114,6 +114,21 @@ __device__ __forceinline__ void lds_load(const void* g, u32 lds) {
 #undef SZ_LDS_LOAD
 }
 
+// A 4-byte global load the compiler keeps no count of (as lds_load's): the caller orders it with wait_vm and must pass the
+// value through load_landed() after the wait and before its first use, which keeps the compiler from moving a use ahead.
+__device__ __forceinline__ float load_f32_uncounted(const float* p) {
+    float v;
+    asm volatile("global_load_dword %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ u32 load_u16_uncounted(const u16* p) {
+    u32 v;
+    asm volatile("global_load_ushort %0, %1, off" : "=v"(v) : "v"(p) : "memory");
+    return v;
+}
+__device__ __forceinline__ void load_landed(float& v) { asm volatile("" : "+v"(v)); }
+__device__ __forceinline__ void load_landed(u32& v) { asm volatile("" : "+v"(v)); }
+
 // s_waitcnt vmcnt(min(n, 63)), nothing else waited for (the counter has 6 bits; waiting for fewer is only earlier).
 template <int n_>
 __device__ __forceinline__ void wait_vm() {
