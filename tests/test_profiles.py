@@ -27,7 +27,9 @@ def test_counters_file_names_kernels_of_the_registry():
         for k, v in entry["kernels"].items():
             assert k in names, (wl, k)
             if "SQ_INSTS_VALU" in v:
-                assert v["busy_cycles"] > 0 and 0.5 < v["clock_ghz"] < 3.0 or v["SQ_WAVES"] < 256, (wl, k, v)
+                # busy cycles are averaged over the 32 shader engines: a launch of fewer waves than the chip has SIMDs leaves
+                # engines idle and reads a low clock, so only launches that fill the chip are held to a plausible one
+                assert v["busy_cycles"] > 0 and 0.5 < v["clock_ghz"] < 3.0 or v["SQ_WAVES"] < 1024, (wl, k, v)
 
 
 class FakeLibrary:
