@@ -1064,8 +1064,9 @@ int32_t sz_verify_round(sz_session* s, uint32_t m, uint64_t u, uint64_t rl, uint
             bool any_exl3 = false;
             for (uint32_t l = 0; l < c.n_layers; l++) any_exl3 = any_exl3 || (s->layers[l].type >= 1021 && s->layers[l].type <= 1033);
             static const bool route_in_launch = std::getenv("SHADOWZERO_ROUTE_IN_LAUNCH") != nullptr;   // the form without the routing launch, for comparisons
-            if (any_exl3 && s->expert_mode == 0 && !route_in_launch) {
+            if (any_exl3 && s->expert_mode == 0 && !route_in_launch && c.n_layers >= 12) {
                 // every layer's router logits are inputs of the round: all of them are routed by one launch before the first layer
+                // (about 10 us, against about 1 us a layer that the selection inside launch 1 costs: not for short rounds)
                 const sz_arg a[] = {P(rl), P(s->plans.ptr), U32(s->plan_stride), U32(c.n_expert), U32(c.top_k), U32(m), U32(c.n_layers)};
                 if (launch("verify_route_layers", (c.n_layers * m + 3) / 4, 1, 1, 256, 0, stream, a)) return 1;
                 ps.plans = s->plans.ptr;

@@ -1039,17 +1039,19 @@ def test_head_top_hands_over_the_sorted_top_64(gpu):
 
 
 # ------------------------------------------------------------------------------------------------- the verify round
-@pytest.mark.parametrize("m,mode", [(4, 0), (1, 0), (2, 0), (8, 0), (4, 1), (4, 2), (1, 2), (8, 2), (5, 1)])
-def test_verify_round_small_with_planted_drafts(gpu, m, mode):
+@pytest.mark.parametrize("m,mode,layers", [(4, 0, 3), (1, 0, 3), (2, 0, 3), (8, 0, 3), (4, 1, 3), (4, 2, 3), (1, 2, 3), (8, 2, 3), (5, 1, 3),
+                                           (4, 0, 12), (1, 0, 12), (8, 0, 12), (3, 2, 12)])
+def test_verify_round_small_with_planted_drafts(gpu, m, mode, layers):
     """Three EXL3 layers of mixed bit rates, a Q8_0 head, and the m - 1 drafts planted so that 0, 1, .. and all of them are
-    accepted; the round replayed as a graph gives the bits of the layer-by-layer calls every time (inside a round all layers
-    are routed by one launch up front and the exact launches read a plan a layer, and a layer's rank-order sum rides the next
-    layer's first launch; a single call selects inside its first launch and sums in a launch of its own).  Token 0 of layer 1
+    accepted; the round replayed as a graph gives the bits of the layer-by-layer calls every time (inside a round of a dozen
+    layers or more all layers are routed by one launch up front and the exact launches read a plan a layer, in a shorter one they
+    select for themselves; a layer's rank-order sum rides the next layer's first launch; a single call selects inside its first
+    launch and sums in a launch of its own).  Token 0 of layer 1
     has fewer finite logits than k (masked experts, session.rs:6205: unused ranks in the plan).  In every mode of the expert
     products: the exact kernels (0) and the two matrix-core forms."""
     rng = np.random.default_rng(77 + m)
     hidden, ff, ne, k, vocab = 512, 256, 12, 4, 3000
-    rates = [2, 3, 4]
+    rates = [2, 3, 4] * (layers // 3)
     s = sz.Session(hidden, ff, ne, k, len(rates), vocab, 8)
     s.set_expert_mode(mode)
     keep_alive, host = [], []
