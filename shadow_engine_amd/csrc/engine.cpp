@@ -587,6 +587,20 @@ int head_argmax_rows(sz_session* s, uint32_t n, uint64_t u, uint64_t logits, uin
     return launch("argmax_merge_parts", n, 1, 1, 256, 0, stream, b);
 }
 
+// The end of a head pass: the rows' arg-max ids out of the partial maxima; with `accept` set (a verify round), the greedy
+// acceptance of the drafts in the same launch.
+struct Accept {
+    uint64_t drafts = 0, out = 0;
+};
+int merge_parts(sz_session* s, uint32_t nparts, uint32_t ts, uint32_t m, uint64_t ids, const Accept* accept, uint64_t stream) {
+    if (accept) {
+        const sz_arg a[] = {P(s->head_part.ptr), U32(nparts), U32(ts), P(ids), U32(m), P(accept->drafts), U32(m - 1), P(accept->out)};
+        return launch("argmax_merge_accept", 1, 1, 1, 1024, 0, stream, a);
+    }
+    const sz_arg b[] = {P(s->head_part.ptr), U32(nparts), U32(ts), P(ids), P(0)};
+    return launch("argmax_merge_parts", m, 1, 1, 256, 0, stream, b);
+}
+
 // The matrix-core head: all m <= 8 rows in one pass over the matrix.  The number of waves a workgroup (each owns at most
 // 512 columns of a row): 4 up to 2048 columns, 6 up to 3072, 8 up to 4096; 0: the shape goes to the scalar kernel.
 uint32_t head_mfma_waves(const sz_session* s) {
@@ -600,7 +614,7 @@ uint32_t head_mfma_waves(const sz_session* s) {
 }
 bool head_mfma_ok(const sz_session* s) { return head_mfma_waves(s) != 0; }
 
-int head_argmax_mfma(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uint64_t ids, uint64_t stream) {
+int head_argmax_mfma(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uint64_t ids, uint64_t stream, const Accept* accept = nullptr) {
     const sz_session_config& c = s->cfg;
     const uint32_t waves = head_mfma_waves(s);
     const uint32_t tiles = (c.vocab + 15) / 16;
@@ -608,8 +622,7 @@ int head_argmax_mfma(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uin
     const sz_arg a[] = {P(s->head_w), P(u), U32(c.hidden), P(logits), U32(c.vocab), P(s->head_part.ptr), U32(c.vocab), U32(c.hidden), U32(m)};
     const char* name = waves == 4 ? "head_q8_0_argmax_mfma" : waves == 6 ? "head_q8_0_argmax_mfma_w6" : "head_q8_0_argmax_mfma_w8";
     if (launch(name, nparts, 1, 1, 64 * waves, 0, stream, a)) return 1;
-    const sz_arg b[] = {P(s->head_part.ptr), U32(nparts), U32(8), P(ids), P(0)};
-    return launch("argmax_merge_parts", m, 1, 1, 256, 0, stream, b);
+    return merge_parts(s, nparts, 8, m, ids, accept, stream);
 }
 
 bool head_is_exl3(const sz_session* s) { return s->head_type >= 1021 && s->head_type <= 1028; }
@@ -641,7 +654,7 @@ bool head_argmax_fused(const sz_session* s) { return s->head_type == SZ_TYPE_Q8_
 
 // An EXL3 head (kernels/exl3.cu:349-461, 610-625 of the reference: rotate the rows once, then one pass over the matrix for all
 // m <= 8 rows): the arg-max ids (0: not wanted) and / or the logits (0: not written).
-int head_exl3(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uint64_t ids, uint64_t stream) {
+int head_exl3(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uint64_t ids, uint64_t stream, const Accept* accept = nullptr) {
     const sz_session_config& c = s->cfg;
     const uint32_t kbs = c.hidden / 128, bits = (uint32_t) s->head_type - 1020;
     {
@@ -653,8 +666,7 @@ int head_exl3(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uint64_t i
     const sz_arg a[] = {P(s->head_w), P(s->head_xa.ptr), P(s->head_inv.ptr), P(logits), U32(c.vocab), P(s->head_part.ptr), U32(c.hidden), U32(c.vocab), U32(m), P(0)};
     if (launch(kn.c_str(), nparts, 1, 1, 256, lds, stream, a)) return 1;
     if (!ids) return 0;
-    const sz_arg b[] = {P(s->head_part.ptr), U32(nparts), U32(8), P(ids), P(0)};
-    return launch("argmax_merge_parts", m, 1, 1, 256, 0, stream, b);
+    return merge_parts(s, nparts, 8, m, ids, accept, stream);
 }
 
 // The number of blocks a row may choose for a hand-off of need_k values (session.rs:5961): three quarters of k_blk, at least
@@ -703,7 +715,8 @@ int head_proxy_sparse(sz_session* s, uint32_t m, uint64_t u, uint32_t need_k, ui
 
 int head_logits(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uint64_t stream);
 
-int head_argmax(sz_session* s, uint32_t m, uint64_t u, uint64_t ids, uint64_t stream) {
+// accept (a verify round): the greedy acceptance after the ids, fused into the merge where the head has one merge for all rows
+int head_argmax(sz_session* s, uint32_t m, uint64_t u, uint64_t ids, uint64_t stream, const Accept* accept = nullptr) {
     if (head_check(s, m, u, "sz_head_argmax")) return 1;
     if (!head_argmax_fused(s)) {
         // mv_cols + topk_rows_at (session.rs:7034-7052): the logits, the largest of every slice of 4096, the largest of those
@@ -712,13 +725,16 @@ int head_argmax(sz_session* s, uint32_t m, uint64_t u, uint64_t ids, uint64_t st
         if (head_logits(s, m, u, s->logits.ptr, stream)) return 1;
         const sz_arg a[] = {P(s->logits.ptr), U32(c.vocab), U32(c.vocab), P(s->head_part.ptr), U32(8)};
         if (launch("argmax_slices", nparts, m, 1, 256, 0, stream, a)) return 1;
-        const sz_arg b[] = {P(s->head_part.ptr), U32(nparts), U32(8), P(ids), P(0)};
-        return launch("argmax_merge_parts", m, 1, 1, 256, 0, stream, b);
+        return merge_parts(s, nparts, 8, m, ids, accept, stream);
     }
-    if (head_is_exl3(s)) return head_exl3(s, m, u, 0, ids, stream);
-    if (head_mfma_ok(s)) return head_argmax_mfma(s, m, u, 0, ids, stream);
+    if (head_is_exl3(s)) return head_exl3(s, m, u, 0, ids, stream, accept);
+    if (head_mfma_ok(s)) return head_argmax_mfma(s, m, u, 0, ids, stream, accept);
     for (uint32_t j0 = 0; j0 < m; j0 += 4) {
         if (head_argmax_rows(s, std::min(4u, m - j0), u + (uint64_t) j0 * s->cfg.hidden * 4, 0, ids + j0 * 4ull, stream)) return 1;
+    }
+    if (accept) {   // the scalar head merges four rows at a time: the acceptance is a launch of its own
+        const sz_arg a[] = {P(ids), P(accept->drafts), U32(m - 1), P(accept->out)};
+        return launch("verify_accept", 1, 1, 1, 64, 0, stream, a);
     }
     return 0;
 }
@@ -1077,9 +1093,8 @@ int32_t sz_verify_round(sz_session* s, uint32_t m, uint64_t u, uint64_t rl, uint
                 if (moe_layer(s, l, m, u + off * c.hidden * 4, rl + off * c.n_expert * 4, sgl + off * 4, y + off * c.hidden * 4, stream, &ps)) return 1;
             }
             if (launch_pending_sum(s, ps, m, stream)) return 1;
-            if (head_argmax(s, m, head_u, out + 8, stream)) return 1;
-            const sz_arg a[] = {P(out + 8), P(drafts), U32(m - 1), P(out)};
-            return launch("verify_accept", 1, 1, 1, 64, 0, stream, a);
+            const Accept acc{drafts, out};
+            return head_argmax(s, m, head_u, out + 8, stream, &acc);
         };
         if (no_graph || !s->use_graph || stream == 0) return record();   // the null stream cannot be captured
         if (sz_capture_begin(stream)) return 1;

@@ -1347,6 +1347,46 @@ extern "C" __global__ void __launch_bounds__(256) argmax_slices(const float* log
     }
 }
 
+// argmax_merge_parts for all m <= 8 rows and the greedy acceptance in one launch (the end of a verify round: one launch and
+// its boundary less): ids[j] as there, then out[0] = keep = 1 + the number of leading drafts d[i] that equal ids[i], out[1] =
+// the bonus token ids[keep - 1] (verify_accept in kernels/moe.hip; engine.rs:2377-2408).  grid 1, block 1024 (128 threads a row).
+extern "C" __global__ void __launch_bounds__(1024) argmax_merge_accept(const u32* part, u32 nparts, u32 ts, u32* ids, u32 m, const u32* drafts,
+                                                                       u32 n_drafts, u32* out) {
+    __shared__ float sv[8][128];
+    __shared__ u32 si[8][128];
+    const u32 j = threadIdx.x >> 7, t = threadIdx.x & 127;
+    float bv = -__builtin_inff();
+    u32 bi = 0xffffffffu;
+    if (j < m)
+        for (u32 p = t; p < nparts; p += 128) argmax_merge(bv, bi, bits_f32(part[((u64) p * ts + j) * 2]), part[((u64) p * ts + j) * 2 + 1]);
+    sv[j][t] = bv;
+    si[j][t] = bi;
+    __syncthreads();
+    for (u32 s = 64; s > 0; s >>= 1) {
+        if (t < s) {
+            float v = sv[j][t];
+            u32 i = si[j][t];
+            argmax_merge(v, i, sv[j][t + s], si[j][t + s]);
+            sv[j][t] = v;
+            si[j][t] = i;
+        }
+        __syncthreads();
+    }
+    if (threadIdx.x < 64) {
+        const u32 i = threadIdx.x;
+        if (i < m) ids[i] = si[i][0];
+        const u32 a = si[min(min(i, n_drafts), 7u)][0];
+        const u32 d = i < n_drafts ? drafts[i] : 0u;
+        const u64 stop = __builtin_amdgcn_ballot_w64(i >= n_drafts || a != d);
+        const u32 first = (u32) __builtin_ctzll(stop);
+        const u32 bonus = __builtin_amdgcn_readlane(a, first);
+        if (i == 0) {
+            out[0] = first + 1;
+            out[1] = bonus;
+        }
+    }
+}
+
 // ids[j] = index of the largest of row j's `nparts` partial maxima part[(p * ts + j) * 2] (ties to the lower index).
 // grid = m, block 256.
 extern "C" __global__ void __launch_bounds__(256) argmax_merge_parts(const u32* part, u32 nparts, u32 ts, u32* ids, float* vals) {
