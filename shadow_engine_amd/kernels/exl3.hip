@@ -1858,18 +1858,23 @@ template <class F>
 __device__ __forceinline__ void xpf_rotate_tile(F&& load4, const u32 (&hop)[2], f32x4 (&rot)[8]) {
 #pragma unroll
     for (int ct = 0; ct < 8; ct++) rot[ct] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
+    // the high and the low parts share one 32-deep matrix instruction: its operands are the sign tile twice and the two parts
+    typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+    typedef u32 u32x4v __attribute__((ext_vector_type(4)));
     typedef u32 u32x2 __attribute__((ext_vector_type(2)));
-    const u32x2 hp = {hop[0], hop[1]}, hn = {hop[0] ^ 0x80008000u, hop[1] ^ 0x80008000u};
+    const f16x8 hp = __builtin_bit_cast(f16x8, u32x4v{hop[0], hop[1], hop[0], hop[1]});
+    const f16x8 hn = __builtin_bit_cast(f16x8, u32x4v{hop[0] ^ 0x80008000u, hop[1] ^ 0x80008000u, hop[0] ^ 0x80008000u, hop[1] ^ 0x80008000u});
 #pragma unroll
     for (int ks = 0; ks < 8; ks++) {
         const f32x4 v = load4(ks);
         const f16x4 av = {(_Float16) v[0], (_Float16) v[1], (_Float16) v[2], (_Float16) v[3]};
         const f16x4 al = {(_Float16) (v[0] - (float) av[0]), (_Float16) (v[1] - (float) av[1]), (_Float16) (v[2] - (float) av[2]), (_Float16) (v[3] - (float) av[3])};
+        const u32x2 ab = __builtin_bit_cast(u32x2, av), lb = __builtin_bit_cast(u32x2, al);
+        const f16x8 parts = __builtin_bit_cast(f16x8, u32x4v{ab[0], ab[1], lb[0], lb[1]});
 #pragma unroll
         for (int ct = 0; ct < 8; ct++) {
             const bool neg = __builtin_popcount(ks & ct) & 1;
-            rot[ct] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, neg ? hn : hp), av, rot[ct], 0, 0, 0);
-            rot[ct] = __builtin_amdgcn_mfma_f32_16x16x16f16(__builtin_bit_cast(f16x4, neg ? hn : hp), al, rot[ct], 0, 0, 0);
+            rot[ct] = __builtin_amdgcn_mfma_f32_16x16x32_f16(neg ? hn : hp, parts, rot[ct], 0, 0, 0);
         }
     }
 }
@@ -1939,6 +1944,55 @@ __device__ __forceinline__ void xpf_wave_products_of(const u32* __restrict__ row
 #pragma unroll
         for (int c = 0; c < 8; c++) acc[T][c] = f32x4{0.0f, 0.0f, 0.0f, 0.0f};
     const u16* xa0 = xa + n16 * 16 + 4 * a;
+    typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+    if constexpr (one_shift && ur == 1) {
+        // Two tile rows a step: a lane's 4 + 4 weights of the rows' tiles are one operand of the 32-deep matrix instruction
+        // (the contraction runs over both rows' 16 inputs; which of them a lane holds does not matter as long as the token
+        // operand is put together the same way), which halves the matrix instructions and their issue slots.
+        typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+        typedef u32 u32x4v __attribute__((ext_vector_type(4)));
+#pragma unroll 1
+        for (u32 i = 0; i < nrows; i += 2) {   // a stream is a whole number of 8-row blocks
+            u32 w1[2][8][2];
+            u32x2 xv[2][NT];
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const u32 r = i + h;
+                exl3_rows_wait<K, D>(r + D > nrows ? r + D - nrows : 0);
+                const u32* row = wb + (r % D) * R::row_words;
+#pragma unroll
+                for (int c = 0; c < 8; c++) {
+                    w1[h][c][0] = row[c * 8 * stride + om1];
+                    w1[h][c][1] = row[c * 8 * stride + op1];
+                }
+#pragma unroll
+                for (int T = 0; T < NT; T++) xv[h][T] = *(const u32x2*) (xa0 + T * XPF_TILE_U16 + r * 256);
+                if (r + D < nrows) {
+                    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): the row's words are in registers, its slot can take the row D further on
+                    exl3_unit_issue<K, D>(row0, pitch, r + D, lane, lds);
+                }
+            }
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                u32 b[2][2];
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const u32 hi = __builtin_amdgcn_alignbit(w1[h][c][0], w1[h][c][1], sh1);
+                    const u32 s0 = __builtin_amdgcn_ubfe(hi, 3 * K, 16), s1 = __builtin_amdgcn_ubfe(hi, 2 * K, 16);
+                    const u32 s2 = __builtin_amdgcn_ubfe(hi, K, 16), s3 = hi & 0xffffu;
+                    b[h][0] = __builtin_bit_cast(u32, exl3_cb2_pair(s0, s1));
+                    b[h][1] = __builtin_bit_cast(u32, exl3_cb2_pair(s2, s3));
+                }
+                const f16x8 bv = __builtin_bit_cast(f16x8, u32x4v{b[0][0], b[0][1], b[1][0], b[1][1]});
+#pragma unroll
+                for (int T = 0; T < NT; T++) {
+                    const f16x8 tv = __builtin_bit_cast(f16x8, u32x4v{xv[0][T][0], xv[0][T][1], xv[1][T][0], xv[1][T][1]});
+                    acc[T][c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(bv, tv, acc[T][c], 0, 0, 0);
+                }
+            }
+        }
+        return;
+    }
 #pragma unroll 1
     for (u32 i = 0; i < nrows; i++) {
         exl3_rows_wait<K, D>(i + D > nrows ? i + D - nrows : 0);
@@ -1953,7 +2007,6 @@ __device__ __forceinline__ void xpf_wave_products_of(const u32* __restrict__ row
                 w0[c][1] = row[c * 8 * stride + op0];
             }
         }
-        typedef u32 u32x2 __attribute__((ext_vector_type(2)));
         f16x4 xv[NT];
 #pragma unroll
         for (int T = 0; T < NT; T++) xv[T] = __builtin_bit_cast(f16x4, *(const u32x2*) (xa0 + T * XPF_TILE_U16 + i * 256));
