@@ -1024,6 +1024,50 @@ __device__ __forceinline__ void exl3_head_kernel(const u8* __restrict__ blob, co
     const bool fed = n < 2 * m;                            // this lane supplies A row n
     const u16* xa0 = aw + (fed ? n : 0) * 128 + 4 * a;
     const u32* wb = wb_all[wave];
+    typedef u32 u32x2 __attribute__((ext_vector_type(2)));
+    if constexpr (one_shift && ur == 1) {
+        // Two tile rows a step on the 32-deep matrix instruction (a lane's 4 + 4 weights of the two rows' tiles against its 4 + 4
+        // A values: the contraction runs over both rows' inputs), half the matrix instructions.  nr is a multiple of 8.
+        typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+        typedef u32 u32x4v __attribute__((ext_vector_type(4)));
+#pragma unroll 1
+        for (u32 i = 0; i < nr; i += 2) {
+            u32 w1[2][8][2];
+            u32x2 xv[2];
+#pragma unroll
+            for (int h = 0; h < 2; h++) {
+                const u32 r = i + h;
+                exl3_rows_wait<K, D>(r + D > nr ? r + D - nr : 0);
+                const u32* row = wb + (r & (D - 1)) * R::row_words;
+#pragma unroll
+                for (int c = 0; c < 8; c++) {
+                    w1[h][c][0] = row[c * 8 * stride + om1];
+                    w1[h][c][1] = row[c * 8 * stride + op1];
+                }
+                xv[h] = *(const u32x2*) (xa0 + (u64) (r >> 3) * nq * 512 + 16 * (r & 7));
+                if (!fed) xv[h] = u32x2{0u, 0u};
+                if (r + D < nr) {
+                    __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0): the row's words are in registers, its slot can take the row D further on
+                    issue(r + D);
+                }
+            }
+            const f16x8 av = __builtin_bit_cast(f16x8, u32x4v{xv[0][0], xv[0][1], xv[1][0], xv[1][1]});
+#pragma unroll
+            for (int c = 0; c < 8; c++) {
+                u32 b[2][2];
+#pragma unroll
+                for (int h = 0; h < 2; h++) {
+                    const u32 hi = __builtin_amdgcn_alignbit(w1[h][c][0], w1[h][c][1], sh1);
+                    const u32 s0 = __builtin_amdgcn_ubfe(hi, 3 * K, 16), s1 = __builtin_amdgcn_ubfe(hi, 2 * K, 16);
+                    const u32 s2 = __builtin_amdgcn_ubfe(hi, K, 16), s3 = hi & 0xffffu;
+                    b[h][0] = __builtin_bit_cast(u32, exl3_cb2_pair(s0, s1));
+                    b[h][1] = __builtin_bit_cast(u32, exl3_cb2_pair(s2, s3));
+                }
+                const f16x8 bv = __builtin_bit_cast(f16x8, u32x4v{b[0][0], b[0][1], b[1][0], b[1][1]});
+                acc[c] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, bv, acc[c], 0, 0, 0);
+            }
+        }
+    } else
 #pragma unroll 1
     for (u32 i = 0; i < nr; i++) {
         exl3_rows_wait<K, D>(i + D > nr ? i + D - nr : 0);
@@ -1038,7 +1082,6 @@ __device__ __forceinline__ void exl3_head_kernel(const u8* __restrict__ blob, co
                 w0[c][1] = row[c * 8 * stride + op0];
             }
         }
-        typedef u32 u32x2 __attribute__((ext_vector_type(2)));
         u32x2 xv = *(const u32x2*) (xa0 + (u64) (i >> 3) * nq * 512 + 16 * (i & 7));
         if (!fed) xv = u32x2{0u, 0u};
         // the row's words are in registers once the reads have returned: its slot can take the row D further on
