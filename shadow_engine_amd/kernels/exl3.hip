@@ -662,8 +662,17 @@ __device__ __forceinline__ void verify_down_kernel(const float* __restrict__ log
     __shared__ u32 sc_all[4][64];      // the wave's 128 f16 scales of down's inputs
     const u32 G = m * k, S = G + m;
     const u32 wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;   // the wave index as a scalar: the index arithmetic on it is the scalar unit's
-    const u32 pair = blockIdx.y;
-    if (logits != nullptr && pair < G && pair % k == 0 && blockIdx.x == 0 && blockIdx.z == 0 && wave == 3) {
+    // Which (pair, column block) this workgroup takes.  Workgroup i of a launch runs on XCD i % 8, each with an L2 of its own,
+    // and the 16 workgroups of a pair all read the pair's partial sums from launch 1: in launch order they sit on all eight
+    // XCDs and the sums are fetched into eight L2s.  Where the shape allows, sets of 8 column blocks of one pair go to one
+    // XCD instead (unit u = the set; the workgroups i with the same i % 8 and the same i / 64 share it), so two L2s fetch them.
+    u32 pair = blockIdx.y, cbx = blockIdx.x;
+    if (gridDim.z == 1 && gridDim.x % 8 == 0 && (gridDim.x / 8 * gridDim.y) % 8 == 0) {
+        const u32 i = blockIdx.y * gridDim.x + blockIdx.x, unit = (i >> 6) * 8 + (i & 7), per = gridDim.x / 8;   // `per` runs a pair
+        pair = unit / per;
+        cbx = ((i >> 3) & 7) * per + unit % per;   // every per-th column block: the run's rows of the trellis spread over the row as the launch order's would
+    }
+    if (logits != nullptr && pair < G && pair % k == 0 && cbx == 0 && blockIdx.z == 0 && wave == 3) {
         // one wave a token: the routing weights and the count, for launch 3 (nothing in this launch reads them)
         const u32 j = pair / k;
         u32 kk;
@@ -698,7 +707,7 @@ __device__ __forceinline__ void verify_down_kernel(const float* __restrict__ log
     float* xw = xw_all[wave];
     u32 svb0 = 0, svb1 = 0;   // wave 0 of a launch without a split over the inputs: down's output scales of the block (needed at the end)
     if (gridDim.z == 1 && wave == 0) {
-        const u16* svh = (const u16*) (bp + 2 * (u64) part + 2 * (u64) ff) + blockIdx.x * 128;
+        const u16* svh = (const u16*) (bp + 2 * (u64) part + 2 * (u64) ff) + cbx * 128;
         svb0 = load_u16_uncounted(svh + lane);
         svb1 = load_u16_uncounted(svh + lane + 64);
     }
@@ -708,7 +717,7 @@ __device__ __forceinline__ void verify_down_kernel(const float* __restrict__ log
         const u32 wb_lds = __builtin_amdgcn_readfirstlane(lds_offset(wb_all[wave]));
         const u8* down = bp + 2 * (u64) part;
         lds_load<4>(down + kb * 256 + lane * 4, sc_lds);                                  // down's input scales
-        const u32* row0 = (const u32*) (down + 2 * (u64) ff + 2 * (u64) hidden + 4) + ((u64) kb * 8 * (hidden / 16) + blockIdx.x * 8) * EXL3_TILE_WORDS(K, H);
+        const u32* row0 = (const u32*) (down + 2 * (u64) ff + 2 * (u64) hidden + 4) + ((u64) kb * 8 * (hidden / 16) + cbx * 8) * EXL3_TILE_WORDS(K, H);
         const u64 pitch = (u64) (hidden / 16) * EXL3_TILE_WORDS(K, H);
         exl3_rows_issue<K, 8, H>(row0, pitch, lane, wb_lds);
         wait_vm<Exl3Rows<K, 8, H>::loads + 1>();   // the partial sums, requested before the burst, have landed
@@ -760,14 +769,14 @@ __device__ __forceinline__ void verify_down_kernel(const float* __restrict__ log
                 a1 += xw_all[w][lane + 64];
             }
             wht128_wave(a0, a1, lane);
-            float* o = dn + (u64) pair * hidden + blockIdx.x * 128;
+            float* o = dn + (u64) pair * hidden + cbx * 128;
             __builtin_nontemporal_store(a0 * sv0, &o[lane]);
             __builtin_nontemporal_store(a1 * sv1, &o[lane + 64]);
         }
     } else if (threadIdx.x < 128) {
         float a = xw_all[0][threadIdx.x];
         for (u32 w = 1; w < nw; w++) a += xw_all[w][threadIdx.x];
-        dn[((u64) pair * gridDim.z + blockIdx.z) * hidden + blockIdx.x * 128 + threadIdx.x] = a;
+        dn[((u64) pair * gridDim.z + blockIdx.z) * hidden + cbx * 128 + threadIdx.x] = a;
     }
 }
 
