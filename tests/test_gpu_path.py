@@ -1461,6 +1461,39 @@ def test_prefill_chunk_of_the_largest_size_equals_its_parts(gpu):
         s.moe_prefill_chunk(0, 16385, x.data_ptr(), dl.data_ptr(), dg.data_ptr(), whole.data_ptr())
 
 
+def test_exl3_prefill_chunk_of_the_largest_size_equals_its_parts(gpu):
+    """The same for EXL3 experts: 16384 tokens in one chunk against chunks of 4096 and 512 (a token's power of two, its
+    rotations and its column of every matrix product do not depend on which other tokens share its work item), and a sample of
+    rows against the exact oracle."""
+    rng = np.random.default_rng(46)
+    tokens, hidden, ff, ne, k, kb = 16384, 512, 256, 48, 6, 3
+    ty = sz.EXL3(kb)
+    dbuf, stride, blobs, sh = build_layer(gpu, rng, ty, hidden, ff, ne, True)
+    s = sz.Session(hidden, ff, ne, k, 1, 0, 8)
+    s.set_layer(0, ty, dbuf.data_ptr(), stride, ty, dbuf.data_ptr() + ne * stride)
+    g = gpu.Generator(device="cuda")
+    g.manual_seed(5)
+    x = gpu.randn((tokens, hidden), device="cuda", generator=g)
+    dl = dev(gpu, synth.zipf_router_logits(rng, tokens, ne))
+    dg = gpu.randn(tokens, device="cuda", generator=g)
+    whole = gpu.zeros((tokens, hidden), dtype=gpu.float32, device="cuda")
+    s.moe_prefill_chunk(0, tokens, x.data_ptr(), dl.data_ptr(), dg.data_ptr(), whole.data_ptr())
+    gpu.cuda.synchronize()
+    want = whole.cpu().numpy()
+    assert np.all(np.isfinite(want)) and np.all(np.abs(want).max(axis=1) > 0)
+    for part in (4096, 512):
+        cut = gpu.zeros((tokens, hidden), dtype=gpu.float32, device="cuda")
+        for t0 in range(0, tokens, part):
+            s.moe_prefill_chunk(0, part, x[t0:].data_ptr(), dl[t0:].data_ptr(), dg[t0:].data_ptr(), cut[t0:].data_ptr())
+        gpu.cuda.synchronize()
+        assert np.array_equal(bits(cut.cpu().numpy()), bits(want)), f"chunks of {part}"
+    xh, lg, sg = x.cpu().numpy(), dl.cpu().numpy(), dg.cpu().numpy()
+    rows = [0, 4097, 9000, tokens - 1]
+    ref, _, _ = oracle_layer(ty, hidden, ff, k, blobs, sh, lg[rows], sg[rows], xh[rows])
+    for i, j in enumerate(rows):
+        assert rel_l2(want[j], ref[i]) <= REL_L2, f"token {j}: {rel_l2(want[j], ref[i])}"
+
+
 def test_config5_full_depth_verify_round(gpu):
     """48 layers of 512 + 1 EXL3 experts at mixed rates (about 29 GB generated in HBM), a 4-token batch, the 151,936-row Q8_0
     head, arg-max and acceptance: token ids and the accepted count exact against the oracle, every layer's output of two
