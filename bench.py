@@ -639,7 +639,7 @@ def main():
     ap.add_argument("--layers", type=int, default=48)
     ap.add_argument("--workload", default="config5", choices=["config1", "config2", "config3", "config4", "config5", "exl3prefill", "exl3head", "exl3top", "stage", "snapshot"])
     ap.add_argument("--rows", type=int, default=4, help="rows of the verify batch (config3, config5, exl3head; the configurations name 4; 1..8)")
-    ap.add_argument("--tokens", type=int, default=512, help="tokens of the prefill chunk (config4 only; the configuration names 512)")
+    ap.add_argument("--tokens", type=int, default=512, help="tokens of the prefill chunk (config4, exl3prefill; the configuration names 512)")
     ap.add_argument("--bits", type=int, default=0, help="bits a weight of the EXL3 head (exl3head, exl3top: 4 unless given) or of the chunk's experts (exl3prefill: 3)")
     ap.add_argument("--expert-mode", type=int, default=0, choices=[0, 1, 2],
                     help="config3, config5: 0 the exact EXL3 expert kernels (the library's default), 1 the matrix-core launches with the codebook's f16 values, 2 with the linearised codebook")
