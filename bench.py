@@ -700,7 +700,7 @@ def main():
     others = None
     if args.workload == "config5" and args.layers == 48 and ROWS == 4 and not args.no_other_configs:
         others = {}
-        for name in ("config1", "config2", "config3", "config4"):
+        for name in ("config1", "config2", "config3", "config4", "exl3prefill"):   # the last: config 4's chunk through the round's kind of experts
             ow = build_workload(name, torch, sz, synth, synth_device, stream, args)
             torch.cuda.synchronize()
             oms, _ = time_steps(ow, stream, sz, torch, 30, 3)
