@@ -225,7 +225,10 @@ def iq3s_prefill(torch, sz, synth, synth_device, stream, tokens=512):
     distinct = int(np.unique(ids).size)
     gu, _, dn = synth.expert_bytes(sz.IQ3_S, HIDDEN, FF)
     w.step_bytes = distinct * (2 * gu + dn) + tokens * (2 * HIDDEN + NE) * 4
-    w.kernel_bytes = {"prefill_gate_up_iq3_s": distinct * 2 * gu + tokens * HIDDEN, "prefill_down_iq3_s": distinct * dn + tokens * TOPK * FF}
+    # gate/up: the experts' two matrices, the tokens' int8 codes and scales in, H's codes and scales out; down: the experts' third
+    # matrix, H in, the pairs' rows of the result out (f32, summed by the combine launch: counted as the EXL3 launches' are)
+    w.kernel_bytes = {"prefill_gate_up_iq3_s": distinct * 2 * gu + tokens * HIDDEN * 9 // 8 + tokens * TOPK * FF * 9 // 8,
+                      "prefill_down_iq3_s": distinct * dn + tokens * TOPK * FF * 9 // 8 + tokens * TOPK * HIDDEN * 4}
     w.kernel_ops = {"prefill_gate_up_iq3_s": 2.0 * tokens * TOPK * 2 * FF * HIDDEN, "prefill_down_iq3_s": 2.0 * tokens * TOPK * FF * HIDDEN}
     w.dtype = "int8 x int8 -> int32 MFMA, f32 scales"
     w.describe = {"workload": "config 4: prefill chunk, %d tokens x hidden 2048 through 512 IQ3_S experts (top-10, Zipf-skewed routing, "
