@@ -1339,7 +1339,8 @@ def test_config4_prefill_chunk_full_size(gpu):
     (5, 40, 256, 256, 6, 2, True),                 # the other rates' lane maps
     (6, 24, 512, 256, 6, 3, True),
     (8, 17, 256, 512, 4, 2, False),
-    (1, 50, 3072, 512, 8, 3, True),                # hidden not a multiple of 512: the last workgroup of the inputs has idle waves
+    (1, 50, 3072, 512, 8, 3, True),                # six workgroups over the inputs, 24 column blocks of the down projection
+    (3, 40, 768, 256, 6, 2, True),                 # hidden not a multiple of 512: the last workgroup over the inputs (and over down's columns) has idle waves
 ])
 def test_exl3_prefill_chunk_matches_the_oracle(gpu, kb, tokens, hidden, ff, ne, k, shared):
     """A prefill chunk through a layer of EXL3 experts (f16 activations on the rows of the matrix instruction, the rotations on
