@@ -1040,7 +1040,7 @@ def test_head_top_hands_over_the_sorted_top_64(gpu):
 
 # ------------------------------------------------------------------------------------------------- the verify round
 @pytest.mark.parametrize("m,mode,layers", [(4, 0, 3), (1, 0, 3), (2, 0, 3), (8, 0, 3), (4, 1, 3), (4, 2, 3), (1, 2, 3), (8, 2, 3), (5, 1, 3),
-                                           (4, 0, 12), (1, 0, 12), (8, 0, 12), (3, 2, 12)])
+                                           (4, 0, 12), (1, 0, 12), (8, 0, 12), (3, 2, 12), (3, 0, 13)])   # 13 x 3: the routing launch's last workgroup has an idle wave
 def test_verify_round_small_with_planted_drafts(gpu, m, mode, layers):
     """Three EXL3 layers of mixed bit rates, a Q8_0 head, and the m - 1 drafts planted so that 0, 1, .. and all of them are
     accepted; the round replayed as a graph gives the bits of the layer-by-layer calls every time (inside a round of a dozen
