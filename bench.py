@@ -126,7 +126,7 @@ def exl3_round(torch, sz, synth, synth_device, stream, L, rates, tag, mode=0):
     pairs = ROWS * (TOPK + 1)                                       # (token, expert) work items, the shared expert included
     act_gu = ROWS * (HIDDEN + NE) * 4 + pairs * 2 * FF * 2 * 4     # u and logits in; two split-K partials of gate and up out
     act_dn = pairs * 2 * FF * 2 * 4 + pairs * HIDDEN * 4           # those partials in; one down output per pair out
-    w.kernel_bytes = {"head_q8_0_argmax": head_bytes + ROWS * HIDDEN * 4, "head_q8_0_argmax_mfma": head_bytes + ROWS * HIDDEN * 4}
+    w.kernel_bytes = {n: head_bytes + ROWS * HIDDEN * 4 for n in ("head_q8_0_argmax", "head_q8_0_argmax_mfma", "head_q8_0_argmax_mfma_n8")}
     for kb in (2, 3, 4):
         for form in ("", "mma_", "mmaw_", "lin_", "linw_"):      # the exact launches and the matrix-core ones (sz_session_set_expert_mode)
             w.kernel_bytes["verify_gate_up_%sexl3_%d" % (form, kb)] = n_sel[kb] * gu_bytes[kb] + act_gu

@@ -621,6 +621,12 @@ int head_argmax_mfma(sz_session* s, uint32_t m, uint64_t u, uint64_t logits, uin
     const uint32_t nparts = std::min<uint32_t>(tiles, waves == 4 ? 512 : 256);       // two workgroups a CU (70 KB of LDS each), one for the wider rows
     const sz_arg a[] = {P(s->head_w), P(u), U32(c.hidden), P(logits), U32(c.vocab), P(s->head_part.ptr), U32(c.vocab), U32(c.hidden), U32(m)};
     const char* name = waves == 4 ? "head_q8_0_argmax_mfma" : waves == 6 ? "head_q8_0_argmax_mfma_w6" : "head_q8_0_argmax_mfma_w8";
+    static const bool four_waves = std::getenv("SHADOWZERO_HEAD_FOUR_WAVES") != nullptr;   // the general form at 2048 columns too, for comparisons
+    if (waves == 4 && c.hidden == 2048 && !four_waves) {
+        // rows of exactly 2048 columns: 8 waves of 256 columns each on the same two tiles of LDS, no per-block checks
+        if (launch("head_q8_0_argmax_mfma_n8", nparts, 1, 1, 512, 0, stream, a)) return 1;
+        return merge_parts(s, nparts, 8, m, ids, accept, stream);
+    }
     if (launch(name, nparts, 1, 1, 64 * waves, 0, stream, a)) return 1;
     return merge_parts(s, nparts, 8, m, ids, accept, stream);
 }

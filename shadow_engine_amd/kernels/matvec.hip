@@ -1159,29 +1159,31 @@ __device__ __forceinline__ void head_tile_issue(const u8* __restrict__ w, u32 ro
     }
 }
 
-// W waves (4, 6 or 8), cols = 512 W at most and a multiple of 64 W.
-template <int W>
+// W waves (4, 6 or 8), cols = CMAX (512 W unless a narrower row is given more waves) at most and a multiple of 64 W.
+template <int W, int CMAX = 512 * W, bool FULL = false>   // FULL: cols == CMAX, every wave owns NBM blocks (no per-block checks: the tile reads of all blocks go out together)
 __device__ __forceinline__ void head_mfma_body(const u8* w, const float* x, u32 xs, float* logits, u32 ls, u32* part, u32 rows, u32 cols, u32 m) {
     __shared__ float s_bv[256];
     __shared__ u32 s_bi[256];
     __shared__ float s_mx[W][8], s_inv[8];   // largest magnitude of a wave's share of every input row; the factor that undoes a row's scale
     const u32 tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63;
+    if constexpr (FULL) cols = CMAX;                      // (the host launches this form for no other width: offsets become constants)
     const u32 rb = cols / 32 * 34, pitch = rb + 16;
-    const u32 kw = cols / W, nbw = kw / 32;               // a wave's columns, and their 32-blocks (<= 16)
+    constexpr int NBM = CMAX / W / 32;                    // the most 32-blocks a wave owns
+    const u32 kw = cols / W, nbw = kw / 32;               // a wave's columns, and their 32-blocks (<= NBM)
     const u32 n16 = lane & 15, g4 = lane >> 4;
-    __shared__ __attribute__((aligned(16))) u8 tiles_lds[2 * 16 * HEAD_PITCH(512 * W)];   // two tiles, 16 * pitch bytes apart
+    __shared__ __attribute__((aligned(16))) u8 tiles_lds[2 * 16 * HEAD_PITCH(CMAX)];   // two tiles, 16 * pitch bytes apart
     __shared__ float red[W][256];
     u8* const tile0 = tiles_lds;
     // the wave's slice of the inputs as B operands: B[k = 4 g4 + i][n = n16], n = 2 j + (0: high part, 1: low part)
-    f16x4 xb[16][2];
+    f16x4 xb[NBM][2];
     {
         const u32 j = n16 >> 1, lowpart = n16 & 1;
         // all 32 loads go out before the first is waited for (clamped to an address that exists where the lane has no
         // input or the block lies past the row: a load behind a branch is waited for on the spot, a round trip each)
-        f32x4 raw[16][2];
+        f32x4 raw[NBM][2];
         const float* xj = x + (u64) min(j, m - 1) * xs + wave * kw + 4 * g4;
 #pragma unroll
-        for (int b = 0; b < 16; b++)
+        for (int b = 0; b < NBM; b++)
 #pragma unroll
             for (int h = 0; h < 2; h++) raw[b][h] = *(const f32x4*) (xj + 32 * min((u32) b, nbw - 1) + 16 * h);
         // every input row is scaled by a power of two that takes its largest magnitude to [2^14, 2^15) before it is split (the
@@ -1189,10 +1191,10 @@ __device__ __forceinline__ void head_mfma_body(const u8* w, const float* x, u32 
         // the low parts of small activations are not lost to f16's subnormal range
         float mxl = 0.0f;
 #pragma unroll
-        for (int b = 0; b < 16; b++)
+        for (int b = 0; b < NBM; b++)
 #pragma unroll
             for (int h = 0; h < 2; h++)
-                if ((u32) b < nbw)
+                if (FULL || (u32) b < nbw)
 #pragma unroll
                     for (int i = 0; i < 4; i++) mxl = fmaxf(mxl, __builtin_fabsf(raw[b][h][i]));   // a NaN is skipped here and shows in the sums
         mxl = fmaxf(mxl, lane_xor<16>(mxl, lane));
@@ -1206,11 +1208,11 @@ __device__ __forceinline__ void head_mfma_body(const u8* w, const float* x, u32 
         pow2_scale_of(f32_bits(mxr), scale, inv);
         if (wave == 0 && g4 == 0 && lowpart == 0) s_inv[j] = inv;
 #pragma unroll
-        for (int b = 0; b < 16; b++)
+        for (int b = 0; b < NBM; b++)
 #pragma unroll
             for (int h = 0; h < 2; h++) {
                 f16x4 v = {0, 0, 0, 0};
-                if ((u32) b < nbw && j < m) {
+                if ((FULL || (u32) b < nbw) && j < m) {
 #pragma unroll
                     for (int i = 0; i < 4; i++) {
                         const float f = raw[b][h][i] * scale;
@@ -1250,8 +1252,8 @@ __device__ __forceinline__ void head_mfma_body(const u8* w, const float* x, u32 
         const u8* drow = tb + (4 * g4) * pitch + wave * nbw * 34;  // scales: rows 4 g4 + r
         float tot[4] = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-        for (int b = 0; b < 16; b++) {
-            if ((u32) b < nbw) {
+        for (int b = 0; b < NBM; b++) {
+            if (FULL || (u32) b < nbw) {
                 const u8* ab = arow + b * 34 + 2 + 4 * g4;
                 const u32 q0 = *(const u16*) ab | ((u32) *(const u16*) (ab + 2) << 16);
                 const u32 q1 = *(const u16*) (ab + 16) | ((u32) *(const u16*) (ab + 18) << 16);
@@ -1304,6 +1306,11 @@ extern "C" __global__ void __launch_bounds__(256, 2) head_q8_0_argmax_mfma(const
 }
 // The same for rows of up to 3072 columns (6 waves, block 384) and up to 4096 (8 waves, block 512): a wave still owns at
 // most 512 columns, the tiles take all of a CU's LDS but for a workgroup's share, so one workgroup a CU.
+// Rows of exactly 2048 columns on 8 waves: the same LDS a workgroup, twice the waves a SIMD to cover the tile reads' latency.
+extern "C" __global__ void __launch_bounds__(512, 2) head_q8_0_argmax_mfma_n8(const u8* w, const float* x, u32 xs, float* logits, u32 ls, u32* part,
+                                                                              u32 rows, u32 cols, u32 m) {
+    head_mfma_body<8, 2048, true>(w, x, xs, logits, ls, part, rows, cols, m);
+}
 extern "C" __global__ void __launch_bounds__(384) head_q8_0_argmax_mfma_w6(const u8* w, const float* x, u32 xs, float* logits, u32 ls, u32* part,
                                                                            u32 rows, u32 cols, u32 m) {
     head_mfma_body<6>(w, x, xs, logits, ls, part, rows, cols, m);

@@ -682,6 +682,7 @@ def planted_head(rng, vocab, hidden, m, winners=None):
 
 @pytest.mark.parametrize("vocab,m,hidden", [(151936, 4, 2048), (1000, 1, 2048), (4099, 8, 2048), (8, 3, 2048),
                                             (3001, 5, 3072), (517, 2, 768), (2048, 3, 4096),    # rows that are not a power of two of 32-weight units
+                                            (3000, 4, 1024), (40000, 8, 1536),                   # four waves a workgroup (2048 columns have a kernel of their own)
                                             (20000, 8, 4096), (20000, 7, 3072), (5000, 2, 2304), (5000, 3, 2560)])   # six and eight waves a workgroup
 def test_head_argmax_and_logits_match_the_oracle(gpu, vocab, m, hidden):
     rng = np.random.default_rng(vocab + m)
