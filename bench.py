@@ -73,15 +73,26 @@ class Workload:
         pass
 
 
+SPACED = True   # --contiguous-experts: the reference's layout, an expert's three blobs back to back
+
+
+def exl3_experts(torch, synth_device, seed, kb):
+    """A layer of EXL3 experts in the layout the stager writes (every trellis on a 128-byte line: sz_layer_spacing), or
+    contiguous: (buffer from the first expert on, stride, gap between an expert's projections)."""
+    if SPACED:
+        return synth_device.exl3_layer(torch, seed, HIDDEN, FF, NE, kb, spaced=True)
+    return (*synth_device.exl3_layer(torch, seed, HIDDEN, FF, NE, kb), 0)
+
+
 def exl3_round(torch, sz, synth, synth_device, stream, L, rates, tag, mode=0):
     w = Workload()
     sess = sz.Session(HIDDEN, FF, NE, TOPK, L, VOCAB, 8)
     sess.set_expert_mode(mode)   # 0: the exact kernels (the default); 1, 2: the matrix-core launches
     layers = []
     for l, kb in enumerate(rates):
-        buf, stride = synth_device.exl3_layer(torch, 1000 + l, HIDDEN, FF, NE, kb)
-        layers.append((buf, stride))
-        sess.set_layer(l, sz.EXL3(kb), buf.data_ptr(), stride, sz.EXL3(kb), buf.data_ptr() + NE * stride)
+        buf, stride, gap = exl3_experts(torch, synth_device, 1000 + l, kb)
+        layers.append((buf, stride, gap))
+        sess.set_layer(l, sz.EXL3(kb), buf.data_ptr(), stride, sz.EXL3(kb), buf.data_ptr() + NE * stride, gap=gap)
     head = synth_device.q8_0_head(torch, 7, VOCAB, HIDDEN)
     sess.set_head(sz.Q8_0, head.data_ptr())
     g = torch.Generator(device="cuda")
@@ -140,7 +151,8 @@ def exl3_round(torch, sz, synth, synth_device, stream, L, rates, tag, mode=0):
     w.dtype = "f32 accumulate over EXL3 f16 codebook weights / Q8_0 int8"
     w.describe = {"workload": "%s: verify round, %d MoE layer%s (hidden 2048, 512 experts + shared, top-10, EXL3 K in %s), %d-token batch, "
                               "Q8_0 lm_head 151936x2048, arg-max, greedy acceptance of %d drafts" % (tag, L, "s" if L > 1 else "", sorted(set(rates)), ROWS, ROWS - 1),
-                  "layers": L, "rows": ROWS, "resident_GB": round(sum(b.numel() for b, _ in layers) / 1e9 + head.numel() / 1e9, 2)}
+                  "layers": L, "rows": ROWS, "resident_GB": round(sum(b.numel() for b, _, _ in layers) / 1e9 + head.numel() / 1e9, 2)}
+    w.describe["expert_layout"] = "every trellis on a 128-byte line (sz_layer_spacing)" if SPACED else "contiguous [gate|up|down]"
     if mode:
         w.describe["expert_mode"] = {1: "matrix cores, the codebook's f16 values", 2: "matrix cores, the linearised codebook"}[mode]
     w.extra = {"accepted_drafts": wrong}
@@ -245,8 +257,8 @@ def exl3_prefill(torch, sz, synth, synth_device, stream, tokens=512, bits=3):
     rows of the matrix instruction (no int8 quantization), the shared expert included."""
     w = Workload()
     sess = sz.Session(HIDDEN, FF, NE, TOPK, 1, 0, 8)
-    buf, stride = synth_device.exl3_layer(torch, 4400, HIDDEN, FF, NE, bits)
-    sess.set_layer(0, sz.EXL3(bits), buf.data_ptr(), stride, sz.EXL3(bits), buf.data_ptr() + NE * stride)
+    buf, stride, gap = exl3_experts(torch, synth_device, 4400, bits)
+    sess.set_layer(0, sz.EXL3(bits), buf.data_ptr(), stride, sz.EXL3(bits), buf.data_ptr() + NE * stride, gap=gap)
     rng = np.random.default_rng(4)
     logits = synth.zipf_router_logits(rng, tokens, NE)
     g = torch.Generator(device="cuda")
@@ -270,9 +282,10 @@ def exl3_prefill(torch, sz, synth, synth_device, stream, tokens=512, bits=3):
     w.dtype = "f32 accumulate over EXL3 f16 codebook weights x f16 activations (matrix cores)"
     w.describe = {"workload": "prefill chunk, %d tokens x hidden 2048 through 512 EXL3 K=%d experts + the shared one (top-10, Zipf-skewed routing, "
                               "%d distinct experts hit), f16 activations" % (tokens, bits, distinct), "rows": tokens, "resident_GB": round(buf.numel() / 1e9, 2)}
+    w.describe["expert_layout"] = "every trellis on a 128-byte line (sz_layer_spacing)" if SPACED else "contiguous [gate|up|down]"
     w.counters_key = "exl3prefill" if (tokens == 512 and bits == 3) else None
     rl_h = logits[:1]
-    w.cpu = ("exl3_token", ((buf, stride), bits, rl_h, x[:1].cpu().numpy(), sgl[:1].cpu().numpy()))
+    w.cpu = ("exl3_token", ((buf, stride, gap), bits, rl_h, x[:1].cpu().numpy(), sgl[:1].cpu().numpy()))
     w.keep = (sess, buf, x, rl, sgl, y)
     return w
 
@@ -389,7 +402,7 @@ def stage_exl3_layer(torch, sz, synth, stream):
     w.extra = {"metric": "checkpoint layer staged into HBM, file bytes a second (reads, pinned buffers, PCIe and the scatter included)", "pcie_inclusive": True}
 
     def check():
-        got = buf[:L.gate_up_bytes].cpu().numpy()
+        got = buf[L.experts_offset:L.experts_offset + L.gate_up_bytes].cpu().numpy()
         want = st.exl3_blob("model.language_model.layers.3.mlp.experts.0.gate_proj")
         if not np.array_equal(got, want):
             raise RuntimeError("the staged layer's first projection is not the checkpoint's")
@@ -546,12 +559,13 @@ def cpu_baseline(kind, args, budget_s=8.0):
     import oracle_lib as O
     hw = int(O.lib().orc_hardware_threads())
     if kind == "exl3_token":
-        (buf, stride), kb, rl0, u0, sgl0 = args
+        (buf, stride, gap), kb, rl0, u0, sgl0 = args
         ty = O.exl3_type(kb)
         shape = O.expert_shape(ty, ty, HIDDEN, FF)
         per_expert = shape.gate_bytes + shape.up_bytes + shape.down_bytes
         ids = np.argsort(-rl0[0].astype(np.float64), kind="stable")[:TOPK]
-        host = {int(e): buf[int(e) * stride:int(e) * stride + per_expert].cpu().numpy() for e in list(ids) + [NE]}
+        from shadow_engine_amd import synth_device
+        host = {int(e): synth_device.expert_host(buf, stride, gap, int(e), (shape.gate_bytes, shape.up_bytes, shape.down_bytes)) for e in list(ids) + [NE]}
         experts = [host.get(e, host[int(ids[0])]) for e in range(NE)]      # only the routed ones are read
         nbytes = (TOPK + 1) * per_expert
         run = lambda t: O.moe_token(shape, experts, TOPK, rl0[0], u0[0], shape, host[NE], float(sgl0[0]), t)
@@ -649,9 +663,14 @@ def main():
     ap.add_argument("--screen", type=int, default=0, help="exl3top: blocks a row of the inexact 2-bit screen (0: the exact hand-off)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true", help="default workload only: do not time configurations 1-4 after it")
+    ap.add_argument("--contiguous-experts", action="store_true",
+                    help="EXL3 experts as the reference keeps them, [gate|up|down] back to back, instead of the stager's layout with every "
+                         "trellis on a 128-byte line (config3, config5, exl3prefill)")
     ap.add_argument("--copy-calibration", type=int, default=0, metavar="BYTES",
                     help="also launch one plain copy of BYTES bytes, for scaling a profile's memory counters")
     args = ap.parse_args()
+    global SPACED
+    SPACED = not args.contiguous_experts
     if args.gpus != 1:
         print("bench.py: this build runs the verify path on ONE GPU (all experts resident in one MI355X's HBM); "
               "--gpus %d is not supported" % args.gpus, file=sys.stderr)

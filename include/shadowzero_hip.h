@@ -153,6 +153,16 @@ void sz_session_free(sz_session*);
  * one type; `shared` (0: none) is the shared expert in the same layout and of type shared_type. */
 int32_t sz_session_set_layer(sz_session*, uint32_t layer, int32_t expert_type, uint64_t experts, uint64_t stride, int32_t shared_type,
                              uint64_t shared);
+/* The same with `gap` bytes (a multiple of 4) between an expert's projections: [gate | gap | up | gap | down], the shared
+ * expert's alike.  No counterpart in the reference, whose experts are contiguous: a layout for this memory.  An EXL3
+ * projection's trellis begins 2 (in + out) + 4 bytes into its blob (exl3.rs:390-393), so in the contiguous layout every row
+ * segment a launch fetches lies 4, 8 or 12 bytes off the 128-byte lines of memory and touches one line more than it fills
+ * (12 to 25 % more bytes fetched).  sz_layer_spacing gives the `lead` (bytes past a 128-byte boundary at which the first
+ * expert, and the shared one, should start) and the `gap` that put every trellis of a layer on a line, given a stride that
+ * is a multiple of 128; both are 0 for GGUF types.  sz_exl3_layer_layout and sz_exl3_stage_layer use them. */
+int32_t sz_session_set_layer_spaced(sz_session*, uint32_t layer, int32_t expert_type, uint64_t experts, uint64_t stride, uint64_t gap,
+                                    int32_t shared_type, uint64_t shared);
+void sz_layer_spacing(int32_t expert_type, uint64_t hidden, uint64_t ff, uint32_t* lead, uint32_t* gap);
 /* output.weight, vocab x hidden: Q8_0, IQ3_S, F32, F16 or BF16 rows, or an EXL3 blob at a whole bit rate (in = hidden, out =
  * vocab, both multiples of 128; the head of an EXL3 checkpoint, session.rs:7179-7187).  The arg-max (sz_head_argmax,
  * sz_verify_round) is fused into the product for Q8_0 and EXL3; the other types go through their logits, kept in a buffer
@@ -357,19 +367,21 @@ int32_t sz_exl3_contiguous(const sz_safetensors*, const char* prefix, uint32_t* 
 uint64_t sz_exl3_blob_len(uint64_t in_features, uint64_t out_features, int32_t type);
 int32_t sz_exl3_read_blob(const sz_safetensors*, const char* prefix, void* host, uint64_t cap);
 
-/* One MoE layer in the device layout sz_session_set_layer and sz_session_set_router take: expert e's [gate | up | down] at
- * e * stride, the shared expert's three at shared_offset, the router at router_offset, the shared expert's gate at
- * gate_offset (a type of -1: the checkpoint has none).  The tensors are `blk.N.ffn_{gate,up,down}_exps.weight`,
+/* One MoE layer in the device layout sz_session_set_layer_spaced and sz_session_set_router take: expert e's
+ * [gate | gap | up | gap | down] at experts_offset + e * stride, the shared expert's three alike at shared_offset, the router
+ * at router_offset, the shared expert's gate at gate_offset (a type of -1: the checkpoint has none).  gap and experts_offset
+ * are sz_layer_spacing's: 0 for a GGUF, what puts every trellis on a 128-byte line for an EXL3 checkpoint.  The tensors are `blk.N.ffn_{gate,up,down}_exps.weight`,
  * `ffn_*_shexp`, `ffn_gate_inp[_shexp]` of a GGUF, and `model.language_model.layers.N.mlp.{experts.E,shared_expert}.*_proj`,
  * `mlp.gate.weight`, `mlp.shared_expert_gate.weight` of an EXL3 checkpoint (exl3_map.rs:128-135). */
 typedef struct {
     int32_t type, shared_type, router_type, gate_type;
-    uint32_t n_expert, reserved;
+    uint32_t n_expert, gap;               /* gap: bytes between an expert's projections */
     uint64_t hidden, ff;
     uint64_t gate_up_bytes, down_bytes;   /* one expert's gate (= up) and down projection */
     uint64_t shared_gate_up_bytes;
     uint64_t stride, shared_offset, router_offset, gate_offset;
     uint64_t bytes;                       /* the whole layer's buffer */
+    uint64_t experts_offset;              /* where expert 0 starts */
 } sz_layer_layout;
 int32_t sz_gguf_layer_layout(const sz_gguf*, uint32_t layer, sz_layer_layout* out);
 /* n_expert = 0: as many experts as the checkpoint has for the layer. */

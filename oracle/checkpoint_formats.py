@@ -471,14 +471,16 @@ def _up256(v):
     return (v + 255) // 256 * 256
 
 
-def layer_image(expert_parts, shared_parts, router, gate):
+def layer_image(expert_parts, shared_parts, router, gate, lead=0, gap=0):
     """The bytes a staged layer must hold: expert_parts[e] = (gate, up, down) byte arrays, shared_parts likewise or None, router
-    and gate byte arrays or None.  Returns (image, mask of the bytes it sets, stride, shared_offset, router_offset, gate_offset)."""
+    and gate byte arrays or None; an expert's projections lie `gap` bytes apart and the first expert (and the shared one)
+    `lead` bytes past a 256-byte boundary (exl3_spacing for an EXL3 layer, 0 and 0 for a GGUF).
+    Returns (image, mask of the bytes it sets, stride, shared_offset, router_offset, gate_offset)."""
     gu, dn = expert_parts[0][0].size, expert_parts[0][2].size
-    stride = _up256(2 * gu + dn)
+    stride = _up256(2 * (gu + gap) + dn)
     ne = len(expert_parts)
-    shared_offset = ne * stride
-    shared_bytes = sum(p.size for p in shared_parts) if shared_parts else 0
+    shared_offset = _up256(lead + ne * stride) + lead
+    shared_bytes = sum(p.size for p in shared_parts) + 2 * gap if shared_parts else 0
     router_offset = _up256(shared_offset + shared_bytes)
     gate_offset = _up256(router_offset + (router.size if router is not None else 0))
     total = _up256(gate_offset + (gate.size if gate is not None else 0))
@@ -490,16 +492,22 @@ def layer_image(expert_parts, shared_parts, router, gate):
         mask[at:at + b.size] = True
 
     for e, (g, u, d) in enumerate(expert_parts):
-        put(e * stride, g)
-        put(e * stride + gu, u)
-        put(e * stride + 2 * gu, d)
+        put(lead + e * stride, g)
+        put(lead + e * stride + gu + gap, u)
+        put(lead + e * stride + 2 * (gu + gap), d)
     if shared_parts:
         at = shared_offset
         for b in shared_parts:
             put(at, b)
-            at += b.size
+            at += b.size + gap
     if router is not None:
         put(router_offset, router)
     if gate is not None:
         put(gate_offset, gate)
     return img, mask, stride, shared_offset, router_offset, gate_offset
+
+
+def exl3_spacing(hidden, ff, blob_bytes):
+    """(lead, gap) that put the trellis of every projection of an EXL3 layer on a 128-byte boundary: the trellis begins
+    2 (in + out) + 4 bytes into a blob (exl3.rs:390-393), projections follow each other blob_bytes + gap apart."""
+    return (128 - (2 * (hidden + ff) + 4) % 128) % 128, (128 - blob_bytes % 128) % 128

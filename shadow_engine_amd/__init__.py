@@ -82,9 +82,9 @@ class StInfo(C.Structure):
 class LayerLayout(C.Structure):
     """sz_layer_layout: where the parts of a staged MoE layer lie in its device buffer."""
     _fields_ = [("type", C.c_int32), ("shared_type", C.c_int32), ("router_type", C.c_int32), ("gate_type", C.c_int32), ("n_expert", C.c_uint32),
-                ("reserved", C.c_uint32), ("hidden", C.c_uint64), ("ff", C.c_uint64), ("gate_up_bytes", C.c_uint64), ("down_bytes", C.c_uint64),
+                ("gap", C.c_uint32), ("hidden", C.c_uint64), ("ff", C.c_uint64), ("gate_up_bytes", C.c_uint64), ("down_bytes", C.c_uint64),
                 ("shared_gate_up_bytes", C.c_uint64), ("stride", C.c_uint64), ("shared_offset", C.c_uint64), ("router_offset", C.c_uint64),
-                ("gate_offset", C.c_uint64), ("bytes", C.c_uint64)]
+                ("gate_offset", C.c_uint64), ("bytes", C.c_uint64), ("experts_offset", C.c_uint64)]
 
 
 _u64, _u32, _i32, _vp = C.c_uint64, C.c_uint32, C.c_int32, C.c_void_p
@@ -143,6 +143,8 @@ _SIGNATURES = {
     "sz_session_new": (_vp, [C.POINTER(SessionConfig)]),
     "sz_session_free": (None, [_vp]),
     "sz_session_set_layer": (_i32, [_vp, _u32, _i32, _u64, _u64, _i32, _u64]),
+    "sz_session_set_layer_spaced": (_i32, [_vp, _u32, _i32, _u64, _u64, _u64, _i32, _u64]),
+    "sz_layer_spacing": (None, [_i32, _u64, _u64, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)]),
     "sz_session_set_head": (_i32, [_vp, _i32, _u64]),
     "sz_session_set_head_proxy": (_i32, [_vp, _u32]),
     "sz_session_set_graph": (_i32, [_vp, _i32]),
@@ -491,8 +493,10 @@ class Session:
         if not self._h:
             raise SzError(last_error())
 
-    def set_layer(self, layer, expert_type, experts_dev, stride, shared_type=0, shared_dev=0):
-        check(lib().sz_session_set_layer(self._h, layer, expert_type, experts_dev, stride, shared_type, shared_dev))
+    def set_layer(self, layer, expert_type, experts_dev, stride, shared_type=0, shared_dev=0, gap=0):
+        """gap: bytes between an expert's projections (0: contiguous [gate|up|down]; layer_spacing() gives the one that puts
+        an EXL3 layer's trellises on 128-byte lines)."""
+        check(lib().sz_session_set_layer_spaced(self._h, layer, expert_type, experts_dev, stride, gap, shared_type, shared_dev))
 
     def set_head(self, ggml_type, w_dev):
         check(lib().sz_session_set_head(self._h, ggml_type, w_dev))
@@ -895,6 +899,14 @@ class SafeTensors:
 
     def stage_exl3_blob(self, prefix, dev, cap, stream=0):
         check(lib().sz_exl3_stage_blob(self._h, prefix.encode(), dev, cap, stream))
+
+
+def layer_spacing(expert_type, hidden, ff):
+    """(lead, gap) of sz_layer_spacing: where a layer's first expert should start past a 128-byte boundary and how far apart an
+    expert's projections should lie for every EXL3 trellis to start on a 128-byte line (0, 0 for GGUF types)."""
+    lead, gap = C.c_uint32(0), C.c_uint32(0)
+    lib().sz_layer_spacing(expert_type, hidden, ff, C.byref(lead), C.byref(gap))
+    return lead.value, gap.value
 
 
 def exl3_blob_len(in_features, out_features, type_id):

@@ -302,6 +302,7 @@ static_assert(sizeof(DenseJob) == 40, "the kernel reads this layout");
 struct SzLayer {
     int type = 0, shared_type = 0;
     uint64_t experts = 0, stride = 0, shared = 0;
+    uint64_t gap = 0; // bytes between an expert's projections (0: the reference's contiguous [gate|up|down])
     DevBuf eaddr;     // u64[3 * ne] then u64[3] for the shared expert
     DevBuf jobs;      // the router launch's job table (set_router)
     uint32_t router_groups = 0;
@@ -454,7 +455,7 @@ int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, ui
         // of the matrix instruction, then the rank-order sum (kernels/exl3.hip, "the verify layer on the matrix cores")
         const MmaPlan mp = mma_plan(m, c.top_k);
         const uint32_t zs_gu = (c.hidden / 128 + 3) / 4, zs_d = exl3_ksplit(c.ff);
-        const uint64_t part = matrix_bytes(f, c.hidden, c.ff);
+        const uint64_t part = matrix_bytes(f, c.hidden, c.ff) + L.gap;   // from one projection of an expert to the next
         if (part >> 32) return fail("sz_moe_layer_verify: a projection of 4 GiB or more");
         const uint32_t nmax = m > 4 ? 8 : 4;
         const uint32_t lds = mma_lds_bytes(f.bits, nmax);
@@ -480,7 +481,7 @@ int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, ui
         // the fused layer: three launches, the work items are the (token, rank) pairs themselves, no plan.  A wave of
         // launch 1 takes one 128-block of the input, 4 waves a workgroup (EXL3_GU_WAVES, EXL3_VERIFY_NB in kernels/exl3.hip).
         const uint32_t S = p.G + m, zs_gu = (c.hidden / 128 + 3) / 4, zs_d = exl3_ksplit(c.ff);
-        const uint64_t part = matrix_bytes(f, c.hidden, c.ff);
+        const uint64_t part = matrix_bytes(f, c.hidden, c.ff) + L.gap;   // from one projection of an expert to the next
         if (part >> 32) return fail("sz_moe_layer_verify: a projection of 4 GiB or more");
         const std::string k1 = "verify_gate_up_" + tag, k2 = "verify_down_" + tag;
         {
@@ -502,7 +503,7 @@ int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, ui
         const uint32_t rpb_gu = rows_per_block(f, c.hidden, m == 1 ? 16 : 32, m == 1 ? 16384 : 32768);
         const uint32_t rpb_d = rows_per_block(f, c.ff, m == 1 ? 32 : 64);
         if (!rpb_gu || !rpb_d) return fail("sz_moe_layer_verify: no kernel for hidden = " + std::to_string(c.hidden) + ", ff = " + std::to_string(c.ff));
-        const uint64_t part = matrix_bytes(f, c.hidden, c.ff);
+        const uint64_t part = matrix_bytes(f, c.hidden, c.ff) + L.gap;   // from one projection of an expert to the next
         if (part >> 32) return fail("sz_moe_layer_verify: a projection of 4 GiB or more");
         const uint32_t rb_gu = c.hidden / f.qk * f.bb, rb_d = c.ff / f.qk * f.bb;
         // One token: two launches.  Launch 1 hands over act = silu(gate) * up and the routing weights, launch 2 owns a row chunk
@@ -795,16 +796,17 @@ void sz_session_free(sz_session* s) {
     delete s;
 }
 
-int32_t sz_session_set_layer(sz_session* s, uint32_t l, int32_t ty, uint64_t experts, uint64_t stride, int32_t shared_type, uint64_t shared) {
+int32_t sz_session_set_layer_spaced(sz_session* s, uint32_t l, int32_t ty, uint64_t experts, uint64_t stride, uint64_t gap, int32_t shared_type, uint64_t shared) {
     clear_error();
     if (!s || l >= s->layers.size()) return fail("sz_session_set_layer: no layer " + std::to_string(l));
     Format f;
     std::string tag;
     if (!format_of(ty, f, tag)) return fail("sz_session_set_layer: ggml type " + std::to_string(ty) + " has no kernels");
     const sz_session_config& c = s->cfg;
-    const uint64_t gu = matrix_bytes(f, c.hidden, c.ff), dn = matrix_bytes(f, c.ff, c.hidden);
+    const uint64_t gu = matrix_bytes(f, c.hidden, c.ff) + gap, dn = matrix_bytes(f, c.ff, c.hidden);   // gu: from a projection to the next
     if (stride < 2 * gu + dn) return fail("sz_session_set_layer: the expert stride is smaller than an expert");
-    if ((experts | stride | shared) & 3) return fail("sz_session_set_layer: expert blobs must be 4-byte aligned");
+    if ((experts | stride | shared | gap) & 3) return fail("sz_session_set_layer: expert blobs must be 4-byte aligned");
+    if (gu >> 32) return fail("sz_session_set_layer: a projection of 4 GiB or more");
     SzLayer& L = s->layers[l];
     // the address table eaddr[part * ne + e] (session.rs:2129-2146), then the shared expert's three parts
     std::vector<uint64_t> tab(3ull * c.n_expert + 3);
@@ -818,7 +820,7 @@ int32_t sz_session_set_layer(sz_session* s, uint32_t l, int32_t ty, uint64_t exp
     std::string tags;
     if (shared) {
         if (!format_of(shared_type, fs, tags)) return fail("sz_session_set_layer: shared type " + std::to_string(shared_type) + " has no kernels");
-        const uint64_t sgu = matrix_bytes(fs, c.hidden, c.ff);
+        const uint64_t sgu = matrix_bytes(fs, c.hidden, c.ff) + gap;
         tab[3ull * c.n_expert] = shared;
         tab[3ull * c.n_expert + 1] = shared + sgu;
         tab[3ull * c.n_expert + 2] = shared + 2 * sgu;
@@ -829,10 +831,32 @@ int32_t sz_session_set_layer(sz_session* s, uint32_t l, int32_t ty, uint64_t exp
     L.experts = experts;
     L.stride = stride;
     L.shared = shared;
+    L.gap = gap;
     L.set = true;
     for (auto& g : s->graphs) sz_graph_destroy(g.second);   // captured address tables may be stale
     s->graphs.clear();
     return 0;
+}
+
+int32_t sz_session_set_layer(sz_session* s, uint32_t l, int32_t ty, uint64_t experts, uint64_t stride, int32_t shared_type, uint64_t shared) {
+    return sz_session_set_layer_spaced(s, l, ty, experts, stride, 0, shared_type, shared);
+}
+
+// Where a layer's experts should lie for their rows to start on 128-byte lines of memory.  An EXL3 projection's trellis
+// begins 2 (in + out) + 4 bytes into its blob (exl3.rs:390-393), and a launch fetches a row of it in segments of 512 to
+// 2048 bytes: 4 bytes off a line, every segment touches one line more than it fills.  With the first blob `lead` bytes past
+// a 128-byte boundary, `gap` bytes between an expert's projections and a stride that is a multiple of 128, every trellis
+// starts on a line.  GGUF rows (34- and 110-byte blocks) have no such boundary: lead and gap 0.
+void sz_layer_spacing(int32_t ty, uint64_t hidden, uint64_t ff, uint32_t* lead, uint32_t* gap) {
+    Format f;
+    std::string tag;
+    uint32_t ld = 0, gp = 0;
+    if (format_of(ty, f, tag) && f.exl3) {
+        ld = (uint32_t) ((128 - (2 * (hidden + ff) + 4) % 128) % 128);
+        gp = (uint32_t) ((128 - matrix_bytes(f, hidden, ff) % 128) % 128);
+    }
+    if (lead) *lead = ld;
+    if (gap) *gap = gp;
 }
 
 int32_t sz_session_set_router(sz_session* s, uint32_t l, int32_t rty, uint64_t rw, int32_t gty, uint64_t gw) {

@@ -460,12 +460,19 @@ uint64_t up256(uint64_t v) { return (v + 255) & ~255ull; }
 
 int dense_type_of(const std::string& dtype) { return dtype == "F32" ? SZ_TYPE_F32 : dtype == "F16" ? SZ_TYPE_F16 : dtype == "BF16" ? SZ_TYPE_BF16 : -1; }
 
-// the layout from the sizes: experts, the shared expert, the router, the shared expert's gate
-void place(sz_layer_layout& L, uint64_t shared_bytes, uint64_t router_bytes, uint64_t gate_bytes) {
-    L.stride = up256(2 * L.gate_up_bytes + L.down_bytes);
-    uint64_t at = (uint64_t) L.n_expert * L.stride;
-    L.shared_offset = at;
-    at = up256(at + shared_bytes);
+// the layout from the sizes: experts, the shared expert (shared_down_bytes: its down projection, 0 without one), the router,
+// the shared expert's gate.  An expert's projections lie L.gap apart and the first one `lead` bytes past a 256-byte
+// boundary (sz_layer_spacing: what puts the rows of an EXL3 trellis on the 128-byte lines of memory; 0 and 0 for a GGUF).
+void place(sz_layer_layout& L, uint64_t shared_down_bytes, uint64_t router_bytes, uint64_t gate_bytes) {
+    uint32_t lead = 0, gap = 0;
+    sz_layer_spacing(L.type, L.hidden, L.ff, &lead, &gap);
+    L.gap = gap;
+    L.experts_offset = lead;
+    L.stride = up256(2 * (L.gate_up_bytes + gap) + L.down_bytes);
+    uint64_t at = up256(lead + (uint64_t) L.n_expert * L.stride);
+    L.shared_offset = at + lead;
+    const uint64_t shared_bytes = shared_down_bytes ? 2 * (L.shared_gate_up_bytes + gap) + shared_down_bytes : 0;
+    at = up256(L.shared_offset + shared_bytes);
     L.router_offset = at;
     at = up256(at + router_bytes);
     L.gate_offset = at;
@@ -513,7 +520,7 @@ int gguf_layer(const sz_gguf* g, uint32_t layer, sz_layer_layout& L, GgufLayer& 
         L.shared_type = (int32_t) sg.type;
         L.shared_gate_up_bytes = sg.nbytes();
         if (su.nbytes() != sg.nbytes()) return fail(p + "ffn_up_shexp.weight: its size differs from the gate's");
-        shared_bytes = 2 * sg.nbytes() + sd.nbytes();
+        shared_bytes = sd.nbytes();   // (the down projection's: place() adds the other two)
     }
     T.router = g->g.tensor(p + "ffn_gate_inp.weight");
     if (T.router) {
@@ -586,7 +593,7 @@ int exl3_layer(const sz_safetensors* st, uint32_t layer, uint32_t n_expert, sz_l
         if (s[1].type != s[0].type || s[2].type != s[0].type) return fail(p + "shared_expert: projections of different types");
         L.shared_type = (int32_t) s[0].type;
         L.shared_gate_up_bytes = exl3_blob_len(L.hidden, L.ff, s[0].bits, s[0].half);
-        shared_bytes = 2 * L.shared_gate_up_bytes + exl3_blob_len(L.ff, L.hidden, s[0].bits, s[0].half);
+        shared_bytes = exl3_blob_len(L.ff, L.hidden, s[0].bits, s[0].half);   // (the down projection's: place() adds the other two)
     }
     T.router = st->st.get(p + "gate.weight");
     if (T.router) {
@@ -633,7 +640,7 @@ int32_t sz_gguf_stage_layer(const sz_gguf* g, uint32_t layer, uint64_t dev, uint
     std::vector<std::string> files;
     for (const GgufShard& s : g->g.shards) files.push_back(s.path);
     std::vector<Piece> ps;
-    const uint64_t part_off[3] = {0, L.gate_up_bytes, 2 * L.gate_up_bytes};
+    const uint64_t part_off[3] = {L.experts_offset, L.experts_offset + L.gate_up_bytes + L.gap, L.experts_offset + 2 * (L.gate_up_bytes + L.gap)};
     // in file order (projection, then expert): the reads of a fused tensor are sequential
     for (int i = 0; i < 3; i++) {
         const uint64_t per = T.e[i]->nbytes() / L.n_expert;
@@ -656,8 +663,8 @@ int32_t sz_gguf_stage_layer(const sz_gguf* g, uint32_t layer, uint64_t dev, uint
     };
     if (T.sh[0]) {
         whole(T.sh[0], L.shared_offset);
-        whole(T.sh[1], L.shared_offset + L.shared_gate_up_bytes);
-        whole(T.sh[2], L.shared_offset + 2 * L.shared_gate_up_bytes);
+        whole(T.sh[1], L.shared_offset + L.shared_gate_up_bytes + L.gap);
+        whole(T.sh[2], L.shared_offset + 2 * (L.shared_gate_up_bytes + L.gap));
     }
     if (T.router) whole(T.router, L.router_offset);
     if (T.gate) whole(T.gate, L.gate_offset);
@@ -697,15 +704,16 @@ int32_t sz_exl3_stage_layer(const sz_safetensors* st, uint32_t layer, uint32_t n
         ps.push_back(std::move(q));
     };
     for (uint32_t e = 0; e < L.n_expert; e++) {
-        blob(T.expert[0][e], L.gate_up_bytes, e * L.stride);
-        blob(T.expert[1][e], L.gate_up_bytes, e * L.stride + L.gate_up_bytes);
-        blob(T.expert[2][e], L.down_bytes, e * L.stride + 2 * L.gate_up_bytes);
+        const uint64_t at = L.experts_offset + e * L.stride, pitch = L.gate_up_bytes + L.gap;
+        blob(T.expert[0][e], L.gate_up_bytes, at);
+        blob(T.expert[1][e], L.gate_up_bytes, at + pitch);
+        blob(T.expert[2][e], L.down_bytes, at + 2 * pitch);
     }
     if (!T.shared[0].empty()) {
-        const uint64_t sgu = L.shared_gate_up_bytes;
+        const uint64_t sgu = L.shared_gate_up_bytes, pitch = sgu + L.gap;
         blob(T.shared[0], sgu, L.shared_offset);
-        blob(T.shared[1], sgu, L.shared_offset + sgu);
-        blob(T.shared[2], sz_exl3_blob_len(L.ff, L.hidden, L.shared_type), L.shared_offset + 2 * sgu);
+        blob(T.shared[1], sgu, L.shared_offset + pitch);
+        blob(T.shared[2], sz_exl3_blob_len(L.ff, L.hidden, L.shared_type), L.shared_offset + 2 * pitch);
     }
     auto whole = [&](const StTensor* t, uint64_t at) {
         Piece q;

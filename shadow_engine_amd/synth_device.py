@@ -10,14 +10,25 @@ import numpy as np
 from . import synth
 
 
-def exl3_layer(torch, seed, hidden, ff, ne, bits):
-    """(buffer uint8[(ne + 1) * stride], stride): experts 0..ne-1 and the shared expert as [gate|up|down] blobs."""
+def exl3_layer(torch, seed, hidden, ff, ne, bits, spaced=False):
+    """(buffer uint8[(ne + 1) * stride], stride): experts 0..ne-1 and the shared expert as [gate|up|down] blobs.
+    spaced: the layout sz_layer_spacing describes instead, every projection's trellis on a 128-byte line of memory - the
+    buffer returned starts at the first expert, an expert's projections lie `gap` bytes apart: (buffer, stride, gap)."""
     g = torch.Generator(device="cuda")
     g.manual_seed(seed)
     gb, ub, db = synth.expert_bytes(synth.exl3_type(bits), hidden, ff)
-    stride = (gb + ub + db + 255) // 256 * 256
+    lead = gap = 0
+    if spaced:
+        import shadow_engine_amd as sz
+        lead, gap = sz.layer_spacing(sz.EXL3(bits), hidden, ff)
+    stride = (gb + ub + db + 2 * gap + 255) // 256 * 256
     n = ne + 1
-    buf = torch.randint(0, 256, (n, stride), dtype=torch.uint8, device="cuda", generator=g)
+    if spaced:
+        full = torch.randint(0, 256, (lead + n * stride,), dtype=torch.uint8, device="cuda", generator=g)
+        assert full.data_ptr() % 256 == 0
+        buf = full[lead:].view(n, stride)
+    else:
+        buf = torch.randint(0, 256, (n, stride), dtype=torch.uint8, device="cuda", generator=g)
     off = 0
     for inf, outf, nbytes in ((hidden, ff, gb), (hidden, ff, ub), (ff, hidden, db)):
         sign = torch.randint(0, 2, (n, inf), device="cuda", generator=g)
@@ -26,8 +37,18 @@ def exl3_layer(torch, seed, hidden, ff, ne, bits):
         buf[:, off:off + 2 * inf] = suh.view(torch.uint8).reshape(n, 2 * inf)
         buf[:, off + 2 * inf:off + 2 * inf + 2 * outf] = svh.view(torch.uint8).reshape(n, 2 * outf)
         buf[:, off + 2 * inf + 2 * outf:off + 2 * inf + 2 * outf + 4] = torch.tensor([1, 0, 0, 0], dtype=torch.uint8, device="cuda")
-        off += nbytes
-    return buf.reshape(-1), stride
+        off += nbytes + gap
+    return (buf.reshape(-1), stride, gap) if spaced else (buf.reshape(-1), stride)
+
+
+def expert_host(buf, stride, gap, e, sizes):
+    """Expert e of a layer buffer as the contiguous [gate|up|down] bytes on the host (sizes: the three projections' bytes)."""
+    import numpy as np
+    at, parts = e * stride, []
+    for n in sizes:
+        parts.append(buf[at:at + n].cpu().numpy())
+        at += n + gap
+    return np.concatenate(parts)
 
 
 def exl3_matrix(torch, seed, inf, outf, bits):

@@ -202,6 +202,7 @@ def test_expert_ranges_and_the_layer_layout_of_a_gguf(tmp_path):
                                                   rw.view(np.uint8).reshape(-1), gw.view(np.uint8).reshape(-1))
     assert (L.type, L.shared_type, L.router_type, L.gate_type, L.n_expert, L.hidden, L.ff) == (sz.IQ3_S, sz.IQ3_S, sz.F32, sz.F32, ne, hidden, ff)
     assert (L.gate_up_bytes, L.down_bytes, L.shared_gate_up_bytes) == (gu, gu, gu)
+    assert (L.gap, L.experts_offset) == (0, 0)                     # a GGUF layer: contiguous, as the reference keeps it
     assert (L.stride, L.shared_offset, L.router_offset, L.gate_offset, L.bytes) == (stride, so, ro, go, img.size)
     with pytest.raises(sz.SzError, match="no tensor blk.1.ffn_gate_exps.weight"):
         g.layer_layout(1)
@@ -388,7 +389,13 @@ def test_the_layer_layout_of_an_exl3_checkpoint(tmp_path):
     st = sz.SafeTensors(d)
     o = F.st_open(st.files())
     L = st.layer_layout(3)
-    img, mask, stride, so, ro, go = F.layer_image(experts, shared, rw.view(np.uint8).reshape(-1), gw.view(np.uint8).reshape(-1))
+    lead, gap = F.exl3_spacing(hidden, ff, experts[0][0].size)
+    assert (lead, gap) == (124, 124) == sz.layer_spacing(sz.EXL3_HALF(2), hidden, ff) and sz.layer_spacing(sz.IQ3_S, hidden, ff) == (0, 0)
+    img, mask, stride, so, ro, go = F.layer_image(experts, shared, rw.view(np.uint8).reshape(-1), gw.view(np.uint8).reshape(-1), lead, gap)
+    assert (L.gap, L.experts_offset) == (gap, lead)
+    # every projection's trellis, 2 (in + out) + 4 bytes into its blob, starts on a 128-byte line of a 256-byte aligned buffer
+    for base, gu in ((L.experts_offset + 2 * L.stride, L.gate_up_bytes), (L.shared_offset, L.shared_gate_up_bytes)):
+        assert all((base + i * (gu + L.gap) + 2 * (hidden + ff) + 4) % 128 == 0 for i in range(3))
     assert (L.type, L.shared_type, L.router_type, L.gate_type, L.n_expert, L.hidden, L.ff) == (sz.EXL3_HALF(2), sz.EXL3(4), sz.BF16, sz.BF16, ne, hidden, ff)
     assert (L.gate_up_bytes, L.down_bytes) == (experts[0][0].size, experts[0][2].size) and L.shared_gate_up_bytes == shared[0].size
     assert (L.stride, L.shared_offset, L.router_offset, L.gate_offset, L.bytes) == (stride, so, ro, go, img.size)
@@ -429,7 +436,8 @@ def run_staged_layer(torch, L, buf, k, m, rng):
     """The MoE block on a staged layer: session, experts, router and gate all from the layout."""
     s = sz.Session(L.hidden, L.ff, L.n_expert, k, 1, 0, 8)
     base = buf.data_ptr()
-    s.set_layer(0, L.type, base, L.stride, L.shared_type if L.shared_type >= 0 else 0, base + L.shared_offset if L.shared_type >= 0 else 0)
+    s.set_layer(0, L.type, base + L.experts_offset, L.stride, L.shared_type if L.shared_type >= 0 else 0,
+                base + L.shared_offset if L.shared_type >= 0 else 0, gap=L.gap)
     s.set_router(0, L.router_type, base + L.router_offset, L.gate_type, base + L.gate_offset)
     u = rng.normal(size=(m, L.hidden)).astype(np.float32)
     du = torch.from_numpy(u).cuda()
@@ -477,7 +485,7 @@ def test_a_layer_staged_from_an_exl3_checkpoint_is_its_blobs_and_runs(gpu, tmp_p
     experts, shared, rw, gw = exl3_checkpoint(d, rng, ty, hidden, ff, ne, shared_ty, scatter=scatter)
     st = sz.SafeTensors(d)
     L, buf = staged(gpu, st, 3)
-    img, mask, *_ = F.layer_image(experts, shared, rw.view(np.uint8).reshape(-1), gw.view(np.uint8).reshape(-1))
+    img, mask, *_ = F.layer_image(experts, shared, rw.view(np.uint8).reshape(-1), gw.view(np.uint8).reshape(-1), *F.exl3_spacing(hidden, ff, experts[0][0].size))
     got = buf.cpu().numpy()
     assert np.array_equal(got[mask], img[mask]) and np.all(got[~mask] == 0xA5)
     u, rl, sgl, y, idx, w = run_staged_layer(gpu, L, buf, k, m, rng)

@@ -277,16 +277,19 @@ def test_unquantized_products_match_the_oracle(gpu, ty, rows, cols):
 
 
 # --------------------------------------------------------------------------------------------------- the MoE layer
-def build_layer(torch, rng, ty, hidden, ff, ne, with_shared=True):
-    """ne experts + one shared expert as one device buffer; returns (device tensor, stride, host blobs, shared blob)."""
+def build_layer(torch, rng, ty, hidden, ff, ne, with_shared=True, lead=0, gap=0):
+    """ne experts + one shared expert as one device buffer; returns (device tensor, stride, host blobs, shared blob).  The
+    first expert starts `lead` bytes into the buffer and an expert's projections lie `gap` bytes apart (0, 0: contiguous
+    [gate|up|down] blobs from the buffer's start); the bytes in between are 0xEE."""
     blobs = [synth.expert_blob(rng, ty, hidden, ff) for _ in range(ne)]
-    stride = (blobs[0].size + 255) // 256 * 256
-    buf = np.zeros((ne + 1) * stride, np.uint8)
-    for e, b in enumerate(blobs):
-        buf[e * stride:e * stride + b.size] = b
+    gb, ub, _ = synth.expert_bytes(ty, hidden, ff)
+    stride = (blobs[0].size + 2 * gap + 255) // 256 * 256
+    buf = np.full(lead + (ne + 1) * stride, 0xEE, np.uint8)
     shared = synth.expert_blob(rng, ty, hidden, ff) if with_shared else None
-    if with_shared:
-        buf[ne * stride:ne * stride + shared.size] = shared
+    for e, b in enumerate(blobs + ([shared] if with_shared else [])):
+        at = lead + e * stride
+        for lo, hi, shift in ((0, gb, 0), (gb, gb + ub, gap), (gb + ub, b.size, 2 * gap)):
+            buf[at + lo + shift:at + hi + shift] = b[lo:hi]
     return dev(torch, buf), stride, blobs, shared
 
 
@@ -478,6 +481,57 @@ def run_moe_layer_case(gpu, ty, hidden, ff, ne, k, m, shared, mode=0):
     gpu.cuda.synchronize()
     assert np.array_equal(bits(dy2.cpu().numpy()), bits(got))
     return (max(rel_l2(got[j], want[j]) for j in range(m)), max(float(np.abs(got[j] - want[j]).max() / np.abs(want[j]).max()) for j in range(m)))
+
+
+@pytest.mark.parametrize("ty,hidden,ff,ne,k,m,mode", [
+    (sz.EXL3(3), 2048, 512, 24, 10, 4, 0), (sz.EXL3(2), 512, 256, 8, 3, 8, 0), (sz.EXL3(4), 512, 1024, 8, 3, 3, 0), (sz.EXL3_HALF(2), 512, 256, 8, 3, 2, 0),
+    (sz.EXL3(3), 512, 256, 8, 3, 5, 1), (sz.EXL3(4), 512, 256, 8, 3, 4, 2),
+    (sz.IQ3_S, 2048, 512, 16, 10, 1, 0), (sz.IQ3_S, 512, 256, 8, 3, 4, 0), (sz.Q8_0, 512, 256, 8, 3, 1, 0), (sz.Q8_0, 512, 256, 8, 3, 6, 0),
+])
+def test_a_layer_with_spaced_projections_gives_the_bits_of_the_contiguous_one(gpu, ty, hidden, ff, ne, k, m, mode):
+    """sz_session_set_layer_spaced: the same experts with a gap between their projections and the first one off the buffer's
+    start (for an EXL3 layer the spacing that puts every trellis on a 128-byte line, for a GGUF layer an arbitrary one) go
+    through the same kernels in the same order: layer outputs, routing and a prefill chunk equal the contiguous layout's bit
+    for bit.  The layouts are also told apart: a stride too small for the gaps is refused."""
+    lead, gap = sz.layer_spacing(ty, hidden, ff) if ty >= 1000 else (36, 60)
+    assert (lead, gap) == ((124, 124) if ty >= 1000 else (36, 60))
+    outs = []
+    for ld, gp in ((0, 0), (lead, gap)):
+        rng = np.random.default_rng(ty + 7 * m)
+        dbuf, stride, blobs, sh = build_layer(gpu, rng, ty, hidden, ff, ne, True, ld, gp)
+        if ty >= 1000 and gp:   # where the trellises lie: 2 (in + out) + 4 bytes into each blob
+            gb = synth.expert_bytes(ty, hidden, ff)[0]
+            assert all((dbuf.data_ptr() + ld + e * stride + i * (gb + gp) + 2 * (hidden + ff) + 4) % 128 == 0 for e in (0, ne) for i in range(3))
+        s = sz.Session(hidden, ff, ne, k, 1, 0, 8)
+        s.set_expert_mode(mode)
+        base = dbuf.data_ptr() + ld
+        if gp:
+            with pytest.raises(sz.SzError, match="stride is smaller"):
+                s.set_layer(0, ty, base, blobs[0].size, ty, base + ne * stride, gap=gp)
+        s.set_layer(0, ty, base, stride, ty, base + ne * stride, gap=gp)
+        u = rng.normal(size=(m, hidden)).astype(np.float32)
+        logits = rng.normal(size=(m, ne)).astype(np.float32)
+        sgl = rng.normal(size=m).astype(np.float32)
+        du, dl, dg = dev(gpu, u), dev(gpu, logits), dev(gpu, sgl)
+        dy = gpu.zeros((m, hidden), dtype=gpu.float32, device="cuda")
+        s.moe_layer_verify(0, m, du.data_ptr(), dl.data_ptr(), dg.data_ptr(), dy.data_ptr())
+        gpu.cuda.synchronize()
+        got = [bits(dy.cpu().numpy()), *s.last_route(m)]
+        if mode == 0 and (ty == sz.IQ3_S or (1020 < ty < 1030)) and hidden % 256 == 0 and ff % 256 == 0 and ff <= 512:
+            tokens = 40
+            x = rng.normal(size=(tokens, hidden)).astype(np.float32)
+            pl = rng.normal(size=(tokens, ne)).astype(np.float32)
+            pg = rng.normal(size=tokens).astype(np.float32)
+            dx, dpl, dpg = dev(gpu, x), dev(gpu, pl), dev(gpu, pg)
+            py = gpu.zeros((tokens, hidden), dtype=gpu.float32, device="cuda")
+            s.moe_prefill_chunk(0, tokens, dx.data_ptr(), dpl.data_ptr(), dpg.data_ptr(), py.data_ptr())
+            gpu.cuda.synchronize()
+            got.append(bits(py.cpu().numpy()))
+        outs.append(got)
+        if (ld, gp) == (0, 0):   # the contiguous run is also right: against the oracle
+            want, widx, ww = oracle_layer(ty, hidden, ff, k, blobs, sh, logits, sgl, u)
+            assert np.array_equal(got[1], widx) and all(rel_l2(dy.cpu().numpy()[j], want[j]) <= MODE_BOUND[mode] for j in range(m))
+    assert len(outs[0]) == len(outs[1]) and all(np.array_equal(a, b) for a, b in zip(outs[0], outs[1]))
 
 
 @pytest.mark.parametrize("ty,hidden,ff,ne,k,m", [
