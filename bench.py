@@ -139,9 +139,9 @@ def exl3_round(torch, sz, synth, synth_device, stream, L, rates, tag, mode=0):
     act_dn = pairs * 2 * FF * 2 * 4 + pairs * HIDDEN * 4           # those partials in; one down output per pair out
     w.kernel_bytes = {n: head_bytes + ROWS * HIDDEN * 4 for n in ("head_q8_0_argmax", "head_q8_0_argmax_mfma", "head_q8_0_argmax_mfma_n8")}
     for kb in (2, 3, 4):
-        for form in ("", "mma_", "mmaw_", "lin_", "linw_"):      # the exact launches and the matrix-core ones (sz_session_set_expert_mode)
-            w.kernel_bytes["verify_gate_up_%sexl3_%d" % (form, kb)] = n_sel[kb] * gu_bytes[kb] + act_gu
-            w.kernel_bytes["verify_down_%sexl3_%d" % (form, kb)] = n_sel[kb] * dn_bytes[kb] + act_dn
+        for form in ("exl3", "mma_exl3", "mmaw_exl3", "lin_exl3", "linw_exl3", "exl3f"):      # the exact launches, the matrix-core ones and the f16-input ones (sz_session_set_expert_mode)
+            w.kernel_bytes["verify_gate_up_%s_%d" % (form, kb)] = n_sel[kb] * gu_bytes[kb] + act_gu
+            w.kernel_bytes["verify_down_%s_%d" % (form, kb)] = n_sel[kb] * dn_bytes[kb] + act_dn
     w.step, w.check, w.set_eager = step, check, (lambda eager: sess.set_graph(not eager))
     w.step_bytes = moe_bytes + head_bytes + act_bytes
     w.counters_key = "config5" if (L == 48 and tag == "config 5" and ROWS == 4) else ("config3" if (tag == "config 3" and ROWS == 4) else None)
@@ -154,7 +154,8 @@ def exl3_round(torch, sz, synth, synth_device, stream, L, rates, tag, mode=0):
                   "layers": L, "rows": ROWS, "resident_GB": round(sum(b.numel() for b, _, _ in layers) / 1e9 + head.numel() / 1e9, 2)}
     w.describe["expert_layout"] = "every trellis on a 128-byte line (sz_layer_spacing)" if SPACED else "contiguous [gate|up|down]"
     if mode:
-        w.describe["expert_mode"] = {1: "matrix cores, the codebook's f16 values", 2: "matrix cores, the linearised codebook"}[mode]
+        w.describe["expert_mode"] = {1: "matrix cores, the codebook's f16 values", 2: "matrix cores, the linearised codebook",
+                                     3: "the exact decode, inputs rounded to f16, two products an instruction"}[mode]
     w.extra = {"accepted_drafts": wrong}
     w.cpu = ("exl3_token", (layers[0], rates[0], rl_h[0], u[0].cpu().numpy(), sgl[0].cpu().numpy()))
     w.keep = (sess, layers, head, u, rl, sgl, hu, y, out, drafts)
@@ -658,8 +659,9 @@ def main():
     ap.add_argument("--rows", type=int, default=4, help="rows of the verify batch (config3, config5, exl3head; the configurations name 4; 1..8)")
     ap.add_argument("--tokens", type=int, default=512, help="tokens of the prefill chunk (config4, exl3prefill; the configuration names 512)")
     ap.add_argument("--bits", type=int, default=0, help="bits a weight of the EXL3 head (exl3head, exl3top: 4 unless given) or of the chunk's experts (exl3prefill: 3)")
-    ap.add_argument("--expert-mode", type=int, default=0, choices=[0, 1, 2],
-                    help="config3, config5: 0 the exact EXL3 expert kernels (the library's default), 1 the matrix-core launches with the codebook's f16 values, 2 with the linearised codebook")
+    ap.add_argument("--expert-mode", type=int, default=0, choices=[0, 1, 2, 3],
+                    help="config3, config5: 0 the exact EXL3 expert kernels (the library's default), 1 the matrix-core launches with the codebook's f16 values, "
+                         "2 with the linearised codebook, 3 the exact launches with their inputs rounded to f16 (two products an instruction)")
     ap.add_argument("--screen", type=int, default=0, help="exl3top: blocks a row of the inexact 2-bit screen (0: the exact hand-off)")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-other-configs", action="store_true", help="default workload only: do not time configurations 1-4 after it")

@@ -187,9 +187,11 @@ int32_t sz_session_set_head_proxy(sz_session*, uint32_t k_blk);
  * multiply-adds in input order, a work item a (token, expert) pair); 1 the matrix cores on the codebook's own f16 values, a
  * work item a distinct expert with its tokens on the rows of the matrix instruction (only the order of the f32 additions and
  * the 22 bits kept of an input differ); 2 the matrix cores on the linearised codebook (a weight's rounding to f16 is skipped:
- * outputs within 1e-3 relative L2 of the exact ones, about 4e-4 measured).  Routing ids, their order and the weights are the
- * same bits in every mode.  Half-integer rates always take the exact kernels.  On an MI355X the exact kernels are the fastest
- * for batches of up to 8 rows.  Environment SHADOWZERO_EXPERT_MODE sets a new session's mode. */
+ * outputs within 1e-3 relative L2 of the exact ones, about 4e-4 measured); 3 the exact kernels' launches and decode with
+ * the rotated inputs rounded to f16, two products an instruction (about 4e-4 as well).  Routing ids, their order and the
+ * weights are the same bits in every mode.  Half-integer rates always take the exact kernels.  On an MI355X modes 1 and 2 are
+ * slower than the exact kernels for batches of up to 8 rows and mode 3 is 1.5 % faster.  Environment SHADOWZERO_EXPERT_MODE
+ * sets a new session's mode. */
 int32_t sz_session_set_expert_mode(sz_session*, int32_t mode);
 /* 0: sz_verify_round launches its kernels one by one instead of replaying a captured graph (default 1). */
 int32_t sz_session_set_graph(sz_session*, int32_t enabled);

@@ -32,6 +32,8 @@ OURS = ("verify_", "decode_", "head_", "argmax_merge", "copy_", "matvec_", "rout
 NAMES = {"config5": ("verify_round_config5", "the default benchmark workload (config 5: 48-layer verify round on a 4-row batch, mixed EXL3 K in {2,3,4}, Q8_0 lm_head)", ""),
          "config5_mode2": ("verify_round_config5_matrix_cores", "bench.py --expert-mode 2 (the config-5 round with the experts on the matrix cores: plan of distinct experts, f16 products, the linearised codebook)",
                            " --expert-mode 2"),
+         "config5_mode3": ("verify_round_config5_f16_inputs", "bench.py --expert-mode 3 (the config-5 round with the exact launches' inputs rounded to f16, two products an instruction)",
+                           " --expert-mode 3"),
          "exl3prefill": ("prefill_chunk_exl3_k3", "bench.py --workload exl3prefill (prefill chunk: 512 tokens through 512 EXL3 K=3 experts + the shared one, f16 matrix cores)", " --workload exl3prefill"),
          "config3": ("verify_layer_and_head_config3", "bench.py --workload config3 (one EXL3 K=3 MoE layer for 4 tokens + Q8_0 head + acceptance)", " --workload config3"),
          "config1": ("matvec_q8_0_config1", "bench.py --workload config1 (one Q8_0 1024 x 2048 matrix-vector product)", " --workload config1"),

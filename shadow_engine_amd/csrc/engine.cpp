@@ -421,7 +421,8 @@ int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, ui
     const PlanLayout p = plan_layout(m, c.top_k);
     // a layer whose sum may ride the next launch takes the plan buffer the pending sum is not reading; a layer routed by the
     // round's routing launch has a plan of its own
-    const bool routed = ride && ride->plans && f.exl3 && s->expert_mode == 0;
+    const bool f16x = s->expert_mode == 3 && f.exl3 && !f.half;   // the exact launches with f16 inputs and two products an instruction
+    const bool routed = ride && ride->plans && f.exl3 && (s->expert_mode == 0 || s->expert_mode == 3);
     const uint64_t plan = routed ? ride->plans + (uint64_t) l * ride->plan_stride
                                  : (ride && ride->active && ride->plan == s->plan.ptr) ? s->plan2.ptr : s->plan.ptr;
     s->last_plan = plan;
@@ -450,7 +451,7 @@ int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, ui
                             U32(c.top_k), U32(m), U32(c.hidden), U32(c.ff), U32(zs_d == 1 ? 0 : zs_d)};
         return launch("verify_combine_exl3", c.hidden / 128, m, 1, zs_d == 1 ? 128 : 1024, 0, stream, a);   // zs_d == 1: launch 2 finished the blocks
     };
-    if (f.exl3 && !f.half && s->expert_mode != 0) {
+    if (f.exl3 && !f.half && (s->expert_mode == 1 || s->expert_mode == 2)) {
         // the matrix-core layer: a plan of the batch's distinct experts, then gate/up and down with an item's tokens on the rows
         // of the matrix instruction, then the rank-order sum (kernels/exl3.hip, "the verify layer on the matrix cores")
         const MmaPlan mp = mma_plan(m, c.top_k);
@@ -483,7 +484,8 @@ int moe_layer(sz_session* s, uint32_t l, uint32_t m, uint64_t u, uint64_t rl, ui
         const uint32_t S = p.G + m, zs_gu = (c.hidden / 128 + 3) / 4, zs_d = exl3_ksplit(c.ff);
         const uint64_t part = matrix_bytes(f, c.hidden, c.ff) + L.gap;   // from one projection of an expert to the next
         if (part >> 32) return fail("sz_moe_layer_verify: a projection of 4 GiB or more");
-        const std::string k1 = "verify_gate_up_" + tag, k2 = "verify_down_" + tag;
+        const std::string ftag = f16x ? "exl3f_" + std::to_string(f.bits) : tag;
+        const std::string k1 = "verify_gate_up_" + ftag, k2 = "verify_down_" + ftag;
         {
             const uint32_t gx = c.ff / 128, extra = (carry_groups + gx * zs_gu - 1) / (gx * zs_gu);   // rows of the grid for a riding sum
             const sz_arg a[] = {P(routed ? 0 : rl), U64(L.experts), U64(L.stride), U64(L.shared), U32((uint32_t) part), P(u), P(plan), P(s->part.ptr),
@@ -770,7 +772,7 @@ sz_session* sz_session_new(const sz_session_config* cfg) {
     sz_session* s = new sz_session();
     s->cfg = c;
     s->layers.resize(c.n_layers);
-    if (const char* e = std::getenv("SHADOWZERO_EXPERT_MODE")) s->expert_mode = std::min(2, std::max(0, std::atoi(e)));
+    if (const char* e = std::getenv("SHADOWZERO_EXPERT_MODE")) s->expert_mode = std::min(3, std::max(0, std::atoi(e)));
     const PlanLayout p = plan_layout(c.max_rows, c.top_k);
     s->GT_max = p.GT;
     const uint64_t ks_gu = exl3_ksplit(c.hidden), ks_d = exl3_ksplit(c.ff);
@@ -976,7 +978,8 @@ uint64_t sz_session_buffer(sz_session* s, int32_t which) {
 int32_t sz_session_set_expert_mode(sz_session* s, int32_t mode) {
     clear_error();
     if (!s) return fail("sz_session_set_expert_mode: null session");
-    if (mode < 0 || mode > 2) return fail("sz_session_set_expert_mode: mode " + std::to_string(mode) + " (0 exact, 1 matrix cores, 2 matrix cores with the linearised codebook)");
+    if (mode < 0 || mode > 3)
+        return fail("sz_session_set_expert_mode: mode " + std::to_string(mode) + " (0 exact, 1 matrix cores, 2 matrix cores with the linearised codebook, 3 exact decode with f16 inputs)");
     if (s->expert_mode != mode) {
         for (auto& g : s->graphs) sz_graph_destroy(g.second);   // a captured round holds the other mode's launches
         s->graphs.clear();
@@ -1110,7 +1113,7 @@ int32_t sz_verify_round(sz_session* s, uint32_t m, uint64_t u, uint64_t rl, uint
             bool any_exl3 = false;
             for (uint32_t l = 0; l < c.n_layers; l++) any_exl3 = any_exl3 || (s->layers[l].type >= 1021 && s->layers[l].type <= 1033);
             static const bool route_in_launch = std::getenv("SHADOWZERO_ROUTE_IN_LAUNCH") != nullptr;   // the form without the routing launch, for comparisons
-            if (any_exl3 && s->expert_mode == 0 && !route_in_launch && c.n_layers >= 12) {
+            if (any_exl3 && (s->expert_mode == 0 || s->expert_mode == 3) && !route_in_launch && c.n_layers >= 12) {
                 // every layer's router logits are inputs of the round: all of them are routed by one launch before the first layer
                 // (about 10 us, against about 1 us a layer that the selection inside launch 1 costs: not for short rounds)
                 const sz_arg a[] = {P(rl), P(s->plans.ptr), U32(s->plan_stride), U32(c.n_expert), U32(c.top_k), U32(m), U32(c.n_layers)};

@@ -303,8 +303,12 @@ __device__ __forceinline__ void exl3_rows_wait(u32 t) {
 // blocks): the first D rows have been requested by exl3_rows_issue, every later row is requested into the ring slot of
 // the row just decoded, so D rows stay in flight until the stream runs out.  xw holds the rotated input (16 values a
 // row) and receives the wave's partial sums of its 128 output columns.
-template <int K, int D = 8, bool H = false>
-__device__ __forceinline__ void exl3_wave_stream(const u32* __restrict__ row0, u64 pitch, u32 rows, const u32* wb, u32 lds, float* xw, u32 lane) {
+// XH: the wave's rotated inputs are f16 (exl3_put_x_f16: pairs of consecutive inputs a word, scaled by a power of two that
+// `unscale` undoes) and two weights meet their two inputs in one v_dot2_f32_f16: 16 instructions a row for the products
+// instead of 32, f32 sums as before, the inputs rounded to 11 bits.
+template <int K, int D = 8, bool H = false, bool XH = false>
+__device__ __forceinline__ void exl3_wave_stream(const u32* __restrict__ row0, u64 pitch, u32 rows, const u32* wb, u32 lds, float* xw, u32 lane,
+                                                 float unscale = 1.0f) {
     typedef Exl3Rows<K, D, H> R;
     constexpr int stride = R::stride, ur = R::unit_rows;
     constexpr int NW = EXL3_NW(K, H);
@@ -346,23 +350,47 @@ __device__ __forceinline__ void exl3_wave_stream(const u32* __restrict__ row0, u
             __builtin_amdgcn_s_waitcnt(0xc07f);   // lgkmcnt(0)
             exl3_unit_issue<K, D, H>(row0, pitch, r + D + 1 - ur, lane, lds);
         }
+        if constexpr (XH) {
+            // the row's 16 inputs as 8 f16 pairs: weights 2 j, 2 j + 1 of the lane meet inputs 2 q + {0, 1} (j even) or 2 q + 8 + {0, 1}
+            // (j odd) of the tile row, q = j / 4
+            typedef u32 u32x4v __attribute__((ext_vector_type(4)));
+            const u32x4v lo = ((const u32x4v*) xw)[2 * r], hi = ((const u32x4v*) xw)[2 * r + 1];
 #pragma unroll
-        for (int q = 0; q < 4; q++) {
-            const float* xr = xw + r * 16 + 2 * q;
-            const float xa[4] = {xr[0], xr[1], xr[8], xr[9]};
+            for (int j = 0; j < 16; j++) {
+                const f16x2 xp = __builtin_bit_cast(f16x2, (j & 1) ? hi[j >> 2] : lo[j >> 2]);
+                if ((j >> 1) & 1) acc1 = __builtin_amdgcn_fdot2(w[j], xp, acc1, false);
+                else acc0 = __builtin_amdgcn_fdot2(w[j], xp, acc0, false);
+            }
+        } else {
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                const int i = 8 * q + e;
-                const int rr = (e & 1) + 2 * ((e >> 1) & 1);
-                if (EXL3_HALF(i)) acc1 = __builtin_fmaf((float) w[i / 2][i % 2], xa[rr], acc1);
-                else acc0 = __builtin_fmaf((float) w[i / 2][i % 2], xa[rr], acc0);
+            for (int q = 0; q < 4; q++) {
+                const float* xr = xw + r * 16 + 2 * q;
+                const float xa[4] = {xr[0], xr[1], xr[8], xr[9]};
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int i = 8 * q + e;
+                    const int rr = (e & 1) + 2 * ((e >> 1) & 1);
+                    if (EXL3_HALF(i)) acc1 = __builtin_fmaf((float) w[i / 2][i % 2], xa[rr], acc1);
+                    else acc0 = __builtin_fmaf((float) w[i / 2][i % 2], xa[rr], acc0);
+                }
             }
         }
     }
     __builtin_amdgcn_wave_barrier();
     const u32 col = (lane >> 3) * 16 + (lane & 7);
-    xw[col] = acc0;
-    xw[col + 8] = acc1;
+    xw[col] = acc0 * unscale;
+    xw[col + 8] = acc1 * unscale;
+}
+
+// A wave's rotated 128-block (the lane holds elements `lane` and `lane + 64`) as f16 in input order at xh[0..127], scaled by
+// the power of two that takes the block's largest magnitude to [2^14, 2^15); returns what undoes the scale.
+__device__ __forceinline__ float exl3_put_x_f16(u16* xh, float a0, float a1, u32 lane) {
+    const float mx = wave_max_f32(fmaxf(__builtin_fabsf(a0), __builtin_fabsf(a1)));
+    float scale, iv;
+    pow2_scale_of(f32_bits(mx), scale, iv);
+    xh[lane] = __builtin_bit_cast(u16, (_Float16) (a0 * scale));
+    xh[lane + 64] = __builtin_bit_cast(u16, (_Float16) (a1 * scale));
+    return iv;
 }
 
 // Group g = blockIdx.y: blob wtab[g], record gtab[17 g] = {n <= 4 (0: unused slot), xi[8], yi[8]}; wave w of the workgroup
@@ -540,7 +568,7 @@ extern "C" __global__ void __launch_bounds__(256) verify_route_layers(const floa
 // sums: gup[((sel * S + pair) * zs + z)][ff], S = m (k + 1), sel 0 = gate, 1 = up, zs = gridDim.z.
 // grid = (ff / 128, 2 S + c, zs), block 64 * EXL3_GU_WAVES; c = 0, or the rows that give (hidden / 128) m more workgroups
 // for the sum of the layer before (cmode).
-template <int K, bool H = false>
+template <int K, bool H = false, bool XH = false>
 __device__ __forceinline__ void verify_gate_up_kernel(const float* __restrict__ logits, u64 ebase, u64 estride, u64 shbase, u32 part,
                                                       const float* __restrict__ u, u8* __restrict__ pbuf, float* __restrict__ gup, u32 ne, u32 k,
                                                       u32 m, u32 hidden, u32 ff, const float* __restrict__ cdn, const u8* __restrict__ cpbuf,
@@ -619,18 +647,24 @@ __device__ __forceinline__ void verify_gate_up_kernel(const float* __restrict__ 
             load_landed(v[b][1]);
         }
         const u16* sc = (const u16*) sc_all[wave];
+        float unscale = 1.0f;
 #pragma unroll
         for (int b = 0; b < NB; b++) {
             if ((u32) b < nb) {
                 float a0 = v[b][0] * f16_to_f32(sc[b * 128 + lane]), a1 = v[b][1] * f16_to_f32(sc[b * 128 + lane + 64]);
                 wht128_wave(a0, a1, lane);
-                xw[b * 128 + lane] = a0;
-                xw[b * 128 + 64 + lane] = a1;
+                if constexpr (XH) {
+                    static_assert(!XH || NB == 1, "the f16 inputs of a wave are one 128-block");
+                    unscale = exl3_put_x_f16((u16*) xw, a0, a1, lane);
+                } else {
+                    xw[b * 128 + lane] = a0;
+                    xw[b * 128 + 64 + lane] = a1;
+                }
             }
         }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        exl3_wave_stream<K, D, H>(row0, pitch, 8 * nb, wb_all[wave], wb_lds, xw, lane);
+        exl3_wave_stream<K, D, H, XH>(row0, pitch, 8 * nb, wb_all[wave], wb_lds, xw, lane, unscale);
     }
     __syncthreads();
     const u32 nw = min((u32) WA, (kbs - min(kbs, blockIdx.z * WA * NB) + NB - 1) / NB);   // waves of this workgroup that had blocks
@@ -653,7 +687,7 @@ __device__ __forceinline__ void verify_gate_up_kernel(const float* __restrict__ 
 // Launch 2: act = silu(gate) * up of the pair, from the sums of launch 1's zs partials, by every wave for the 128-block of
 // act it is about to use (16-fold redundant work of a hundred operations, instead of a launch), then the down
 // product's partial sums: dn[pair * gridDim.z + z][hidden].  grid = (hidden / 128, S, ceil(ff / 512)), block 256.
-template <int K, bool H = false>
+template <int K, bool H = false, bool XH = false>
 __device__ __forceinline__ void verify_down_kernel(const float* __restrict__ logits, u64 ebase, u64 estride, u64 shbase, u32 part,
                                                    u8* __restrict__ pbuf, const float* __restrict__ gup, float* __restrict__ dn, u32 ne, u32 k, u32 m,
                                                    u32 hidden, u32 ff, u32 zs) {
@@ -747,11 +781,16 @@ __device__ __forceinline__ void verify_down_kernel(const float* __restrict__ log
         float a0 = (siluf_ref(g0) * u0) * f16_to_f32(suh[lane]);
         float a1 = (siluf_ref(g1) * u1) * f16_to_f32(suh[lane + 64]);
         wht128_wave(a0, a1, lane);
-        xw[lane] = a0;
-        xw[64 + lane] = a1;
+        float unscale = 1.0f;
+        if constexpr (XH) {
+            unscale = exl3_put_x_f16((u16*) xw, a0, a1, lane);
+        } else {
+            xw[lane] = a0;
+            xw[64 + lane] = a1;
+        }
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
-        exl3_wave_stream<K, 8, H>(row0, pitch, 8, wb_all[wave], wb_lds, xw, lane);
+        exl3_wave_stream<K, 8, H, XH>(row0, pitch, 8, wb_all[wave], wb_lds, xw, lane, unscale);
     }
     __syncthreads();
     const u32 nw = min(4u, kbs - blockIdx.z * 4);
@@ -797,6 +836,20 @@ __device__ __forceinline__ void verify_down_kernel(const float* __restrict__ log
         verify_down_kernel<K>(logits, ebase, estride, shbase, part, pbuf, gup, dn, ne, k, m, hidden, ff, zs);                             \
     }
 
+// The same launches with the rotated inputs rounded to f16 and two products an instruction (session expert mode 3).
+#define EXL3_VERIFY_F16_ENTRIES(K)                                                                                                        \
+    extern "C" __global__ void __launch_bounds__(64 * EXL3_GU_WAVES, EXL3_GU_OCC(K)) verify_gate_up_exl3f_##K(const float* logits, u64 ebase, u64 estride, u64 shbase, u32 part, \
+                                                                                  const float* u, u8* pbuf, float* gup, u32 ne, u32 k, u32 m, \
+                                                                                  u32 hidden, u32 ff, const float* cdn, const u8* cpbuf,      \
+                                                                                  const float* cgl, float* cy, u32 cmode) {                   \
+        verify_gate_up_kernel<K, false, true>(logits, ebase, estride, shbase, part, u, pbuf, gup, ne, k, m, hidden, ff, cdn, cpbuf, cgl, cy, cmode); \
+    }                                                                                                                                     \
+    extern "C" __global__ void __launch_bounds__(256, EXL3_VERIFY_WAVES(K)) verify_down_exl3f_##K(const float* logits, u64 ebase, u64 estride, u64 shbase, u32 part,   \
+                                                                               u8* pbuf, const float* gup, float* dn, u32 ne, u32 k, u32 m,   \
+                                                                               u32 hidden, u32 ff, u32 zs) {                                  \
+        verify_down_kernel<K, false, true>(logits, ebase, estride, shbase, part, pbuf, gup, dn, ne, k, m, hidden, ff, zs);                \
+    }
+
 // K + 1/2 bits a weight: the LDS and register budget of the next whole rate
 #define EXL3_VERIFY_HALF_ENTRIES(K)                                                                                                       \
     extern "C" __global__ void __launch_bounds__(64 * EXL3_GU_WAVES, EXL3_GU_OCC(K + 1)) verify_gate_up_exl3h_##K(const float* logits, u64 ebase, u64 estride, u64 shbase, u32 part, \
@@ -814,6 +867,15 @@ __device__ __forceinline__ void verify_down_kernel(const float* __restrict__ log
 EXL3_VERIFY_HALF_ENTRIES(1)
 EXL3_VERIFY_HALF_ENTRIES(2)
 EXL3_VERIFY_HALF_ENTRIES(3)
+
+EXL3_VERIFY_F16_ENTRIES(1)
+EXL3_VERIFY_F16_ENTRIES(2)
+EXL3_VERIFY_F16_ENTRIES(3)
+EXL3_VERIFY_F16_ENTRIES(4)
+EXL3_VERIFY_F16_ENTRIES(5)
+EXL3_VERIFY_F16_ENTRIES(6)
+EXL3_VERIFY_F16_ENTRIES(7)
+EXL3_VERIFY_F16_ENTRIES(8)
 
 EXL3_VERIFY_ENTRIES(1)
 EXL3_VERIFY_ENTRIES(2)
