@@ -1231,7 +1231,8 @@ int32_t sz_moe_prefill_chunk(sz_session* s, uint32_t l, uint32_t tokens, uint64_
     {
         const sz_arg a[] = {P(L.eaddr.ptr), P(sh), P(pb.offs.ptr), P(pb.list.ptr), P(pb.items.ptr), P(pb.xq.ptr), P(pb.xd.ptr), P(pb.hq.ptr), P(pb.hd.ptr),
                             U32(c.n_expert), U32(c.top_k), U32((uint32_t) np), U32(c.hidden), U32(c.ff)};
-        if (launch("prefill_gate_up_iq3_s", c.ff / 64, (uint32_t) max_items, 1, 256, 0, stream, a)) return 1;
+        static const bool w4 = std::getenv("SHADOWZERO_PREFILL_FOUR_WAVES") != nullptr;   // the four-wave form, for comparisons
+        if (launch(w4 ? "prefill_gate_up_iq3_s_w4" : "prefill_gate_up_iq3_s", c.ff / 64, (uint32_t) max_items, 1, w4 ? 256 : 512, 0, stream, a)) return 1;
     }
     {
         // a workgroup takes 4 (else 2, else 1) blocks of 64 rows in turn: the two chunks of one block are too little work for its set-up

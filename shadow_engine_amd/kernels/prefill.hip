@@ -229,17 +229,18 @@ __device__ __forceinline__ void iq3s_scales_to_strip(const u8* blk, u32 n, u32 k
 // The int8 activations and their scales of TOK pairs (32 or 64) for k in [k0, k0 + 256).  Token t's 16-byte column c lands at
 // slot c ^ (t & 15) of its row: the 16 tokens of an MFMA tile then read the same column from 16 different bank groups.
 // `rows` (LDS): the row of q and d every pair reads; a pair past the item's end names row 0, whose products are dropped.
-template <int TOK>
+template <int TOK, int NWV = 4>   // NWV: the waves that share the chunk's loads
 __device__ __forceinline__ void pf_issue_a(const i8* __restrict__ q, const float* __restrict__ d, const u32* rows, u32 cols, u32 k0, u32 lds_a,
                                            u32 lds_d, u32 wave, u32 lane) {
+    static_assert((TOK / 8) % NWV == 0, "every wave the same number of load instructions");
 #pragma unroll
-    for (int it = 0; it < TOK / 16; it++) {               // TOK / 4 instructions a chunk: 4 tokens each
-        const u32 j = wave * (TOK / 16) + it, t = 4 * j + (lane >> 4), c = (lane & 15) ^ (t & 15);
+    for (int it = 0; it < TOK / 4 / NWV; it++) {          // TOK / 4 instructions a chunk: 4 tokens each
+        const u32 j = wave * (TOK / 4 / NWV) + it, t = 4 * j + (lane >> 4), c = (lane & 15) ^ (t & 15);
         lds_load<16>(q + (u64) rows[t] * cols + k0 + 16 * c, lds_a + j * 1024);
     }
 #pragma unroll
-    for (int it = 0; it < TOK / 32; it++) {               // TOK / 8 instructions: 64 of the 8 x TOK scales each
-        const u32 j = wave * (TOK / 32) + it, i = j * 64 + lane, g = i / TOK, t = i % TOK;
+    for (int it = 0; it < TOK / 8 / NWV; it++) {          // TOK / 8 instructions: 64 of the 8 x TOK scales each
+        const u32 j = wave * (TOK / 8 / NWV) + it, i = j * 64 + lane, g = i / TOK, t = i % TOK;
         lds_load<4>(d + (u64) rows[t] * (cols / 32) + k0 / 32 + g, lds_d + j * 256);
     }
 }
@@ -250,27 +251,36 @@ __device__ __forceinline__ void pf_issue_a(const i8* __restrict__ q, const float
 // word and its last one ends on one (a row is a multiple of 4 bytes, or rows come in even numbers).
 // w = the first of the 64 rows, rb = bytes a row.
 __device__ __forceinline__ u32 pf_shift(const u8* w, u32 rb, u32 c, u32 row) { return (u32) ((u64) (w + (u64) row * rb + c * 110) & 2); }
+template <int NWV = 4>
 __device__ __forceinline__ void pf_issue_w(const u8* __restrict__ w, u32 rb, u32 c, u32 lds_w, u32 wave, u32 lane) {
 #pragma unroll
-    for (int it = 0; it < 7; it++) {                      // 28 instructions a chunk and matrix: 64 rows x 28 words
-        const u32 j = wave * 7 + it, i = j * 64 + lane, row = i / 28, dw = i % 28;
-        const u8* a = w + (u64) row * rb + c * 110;
-        lds_load<4>(a - ((u64) a & 2) + 4 * dw, lds_w + j * 256);
+    for (int it = 0; it < (28 + NWV - 1) / NWV; it++) {   // 28 instructions a chunk and matrix: 64 rows x 28 words
+        const u32 j = NWV == 4 ? wave * 7 + it : wave + NWV * it;
+        if (j < 28) {                                     // (wave-uniform)
+            const u32 i = j * 64 + lane, row = i / 28, dw = i % 28;
+            const u8* a = w + (u64) row * rb + c * 110;
+            lds_load<4>(a - ((u64) a & 2) + 4 * dw, lds_w + j * 256);
+        }
     }
 }
 
 // One staged chunk's products: for each of its 8 sub-blocks the lane's 8 weights of its row (gate and up, or down) against
 // the first T token tiles, every tile's exact int32 sums scaled and added in f32 (a fused multiply-add a sum, in sub-block
 // order).  aq, ad: the chunk's activations and their scales; bg, bu, bd: the lane's row's block in LDS.
-template <int T, int TOK>
+template <int V> struct pf_int { static constexpr int value = V; };
+
+// NG sub-blocks from G0 on (8 from 0: the whole block; 4 from 0 or 4: a wave's half where two waves share a row group).
+template <int T, int TOK, int NG = 8, int G0 = 0>
 __device__ __forceinline__ void pf_products_gu(float (&accg)[PF_TILES][4], float (&accu)[PF_TILES][4], const u8* aq, const float* ad, const u8* bg, const u8* bu,
                                                u32 n, u32 kq, float* sw) {
+    constexpr u32 g0 = G0;
     iq3s_scales_to_strip(bg, n, kq, sw);
     iq3s_scales_to_strip(bu, n, kq, sw + 128);
     __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
     __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (u32 g = 0; g < 8; g++) {
+    for (u32 gg = 0; gg < NG; gg++) {
+        const u32 g = g0 + gg;
         const float swg = sw[g * 16 + n], swu = sw[128 + g * 16 + n];
         const u64 b_g = iq3s_int8x8(bg, g, kq), b_u = iq3s_int8x8(bu, g, kq);
         const u32 col = ((2 * g + (kq >> 1)) ^ n) * 16 + 8 * (kq & 1);   // where this lane's 8 activations of a token lie in its row
@@ -311,30 +321,34 @@ __device__ __forceinline__ void pf_products_d(float (&acc)[TOK / 16][4], const u
     }
 }
 
-// Work item blockIdx.y = (expert, first position) from prefill_group: gate and up rows [64 blockIdx.x + 16 wave, +16) of
+// Work item blockIdx.y = (expert, first position) from prefill_group: gate and up rows [64 blockIdx.x + 16 (wave & 3), +16) of
 // the expert against up to 64 of its pairs' tokens, SwiGLU (silu in f32, cpu_expert.rs:217), and H re-quantized per 32
 // features: hq[pair][ff], hd[pair][ff / 32].  eaddr[part * ne + e] / sh_addr[part] as in the planner's kernels.
-// grid = (ff / 64, the bound on the number of items), block 256.
-extern "C" __global__ void __launch_bounds__(256, 2) prefill_gate_up_iq3_s(const u64* eaddr, const u64* sh_addr, const u32* offs, const u32* list,
-                                                                        const u32* items, const i8* xq, const float* xd, i8* hq, float* hd, u32 ne,
-                                                                        u32 k, u32 npairs, u32 hidden, u32 ff) {
+// grid = (ff / 64, the bound on the number of items), block 64 NWV.
+// NWV = 4: wave w rows 16 w .. 16 w + 15, all 8 sub-blocks of a chunk's block.  NWV = 8 (block 512): waves w and w + 4 share
+// the rows 16 (w & 3) .. and take sub-blocks 0..3 and 4..7 of every block; their partial sums are added at the end (the same
+// LDS a workgroup, twice the waves a SIMD to cover the LDS reads and the barriers of a chunk).
+template <int NWV>
+__device__ __forceinline__ void prefill_gate_up_iq3_s_body(const u64* eaddr, const u64* sh_addr, const u32* offs, const u32* list, const u32* items,
+                                                           const i8* xq, const float* xd, i8* hq, float* hd, u32 ne, u32 k, u32 npairs, u32 hidden, u32 ff) {
     // two buffers of a chunk: activations | gate rows | up rows | activation scales; afterwards the item's 64 x 64 block of H
     constexpr u32 AB = PF_AB(PF_TOK), BUF = AB + 2 * PF_WB + PF_DB(PF_TOK);
     __shared__ __attribute__((aligned(16))) u8 stage[2 * BUF];
     __shared__ u32 s_rows[PF_TOK], s_pairs[PF_TOK];
-    __shared__ float s_sw[4][256];   // a wave's strip of sub-block scales: gate [8][16], up [8][16]
-    static_assert(sizeof(stage) >= PF_TOK * 65 * sizeof(float), "H reuses the staging area");
+    __shared__ float s_sw[NWV][256];   // a wave's strip of sub-block scales: gate [8][16], up [8][16]
+    static_assert(sizeof(stage) >= 3 * PF_TOK * 65 * sizeof(float), "H and the second half's partial sums reuse the staging area");
     float (*hs)[65] = (float (*)[65]) stage;
     const u32 tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
     const u32 n = lane & 15, kq = lane >> 4;
-    const u32 lrow = wave * 16 + n;                      // the lane's weight row inside the workgroup's 64
+    const u32 rw = wave & 3, kh = wave >> 2;             // the wave's row group; which half of the sub-blocks (NWV = 8)
+    const u32 lrow = rw * 16 + n;                        // the lane's weight row inside the workgroup's 64
     const u32 rb = hidden / 256 * 110, rbx = blockIdx.x;
     const u32 lds0 = __builtin_amdgcn_readfirstlane(lds_offset(stage));
     if (blockIdx.y >= items[0]) return;
     const u32 e = items[1 + 2 * blockIdx.y], t0 = items[2 + 2 * blockIdx.y];
     if (e == ne && !sh_addr) return;
     const u32 first = offs[e], nt = min((u32) PF_TOK, offs[e + 1] - first - t0);
-    pf_tables(tid);
+    if (tid < 256) pf_tables(tid);
     const u8* wg = (const u8*) (e < ne ? eaddr[e] : sh_addr[0]) + (u64) rbx * 64 * rb;
     const u8* wu = (const u8*) (e < ne ? eaddr[(u64) ne + e] : sh_addr[1]) + (u64) rbx * 64 * rb;
     if (tid < PF_TOK) {
@@ -350,37 +364,86 @@ extern "C" __global__ void __launch_bounds__(256, 2) prefill_gate_up_iq3_s(const
     __syncthreads();   // s_rows and the tables are written
     auto issue = [&](u32 c) {
         const u32 base = lds0 + (c & 1) * BUF;
-        pf_issue_a<PF_TOK>(xq, xd, s_rows, hidden, c * PF_KC, base, base + AB + 2 * PF_WB, wave, lane);
-        pf_issue_w(wg, rb, c, base + AB, wave, lane);
-        pf_issue_w(wu, rb, c, base + AB + PF_WB, wave, lane);
+        pf_issue_a<PF_TOK, NWV>(xq, xd, s_rows, hidden, c * PF_KC, base, base + AB + 2 * PF_WB, wave, lane);
+        pf_issue_w<NWV>(wg, rb, c, base + AB, wave, lane);
+        pf_issue_w<NWV>(wu, rb, c, base + AB + PF_WB, wave, lane);
     };
     const u32 nc = hidden / PF_KC;
-    issue(0);
-    for (u32 c = 0; c < nc; c++) {
-        wait_vm<0>();
-        __syncthreads();   // chunk c is in LDS, from every wave; the products of chunk c - 1 are done, so its buffer is free
-        if (c + 1 < nc) issue(c + 1);
-        const u8* buf = stage + (c & 1) * BUF;
-        const u8* aq = buf;
-        const float* ad = (const float*) (buf + AB + 2 * PF_WB);
-        const u8* bg = buf + AB + lrow * PF_WS + pf_shift(wg, rb, c, lrow);
-        const u8* bu = buf + AB + PF_WB + lrow * PF_WS + pf_shift(wu, rb, c, lrow);
-        switch ((nt + 15) / 16) {   // straight-line code for the item's number of token tiles: the scheduler overlaps one tile's loads and
-                                    // matrix instructions with the scaling of the tile before it
-            case 1: pf_products_gu<1, PF_TOK>(accg, accu, aq, ad, bg, bu, n, kq, s_sw[wave]); break;
-#if PF_TILES > 2
-            case 2: pf_products_gu<2, PF_TOK>(accg, accu, aq, ad, bg, bu, n, kq, s_sw[wave]); break;
-            case 3: pf_products_gu<3, PF_TOK>(accg, accu, aq, ad, bg, bu, n, kq, s_sw[wave]); break;
-#endif
-            default: pf_products_gu<PF_TILES, PF_TOK>(accg, accu, aq, ad, bg, bu, n, kq, s_sw[wave]); break;
+    constexpr int NG = NWV == 8 ? 4 : 8;
+    // The loop over the chunks, straight-line code for the item's number of token tiles T (the scheduler overlaps one tile's
+    // loads and matrix instructions with the scaling of the tile before it) and, with 8 waves, for the wave's half of the
+    // sub-blocks: chosen once, outside the loop, so that only T tiles' sums are live in it.
+    auto chunks = [&](auto tiles, auto half) {
+        constexpr int T = decltype(tiles)::value, G0 = decltype(half)::value;
+        float ag[PF_TILES][4], au[PF_TILES][4];
+#pragma unroll
+        for (int a = 0; a < T; a++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) ag[a][r] = au[a][r] = 0.0f;
+        issue(0);
+        for (u32 c = 0; c < nc; c++) {
+            wait_vm<0>();
+            __syncthreads();   // chunk c is in LDS, from every wave; the products of chunk c - 1 are done, so its buffer is free
+            if (c + 1 < nc) issue(c + 1);
+            const u8* buf = stage + (c & 1) * BUF;
+            const u8* aq = buf;
+            const float* ad = (const float*) (buf + AB + 2 * PF_WB);
+            const u8* bg = buf + AB + lrow * PF_WS + pf_shift(wg, rb, c, lrow);
+            const u8* bu = buf + AB + PF_WB + lrow * PF_WS + pf_shift(wu, rb, c, lrow);
+            pf_products_gu<T, PF_TOK, NG, G0>(ag, au, aq, ad, bg, bu, n, kq, s_sw[wave]);
         }
+#pragma unroll
+        for (int a = 0; a < T; a++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) {
+                accg[a][r] = ag[a][r];
+                accu[a][r] = au[a][r];
+            }
+    };
+    auto halves = [&](auto tiles) {
+        if (NWV == 8 && kh == 1) chunks(tiles, pf_int<4>{});
+        else chunks(tiles, pf_int<0>{});
+    };
+    switch ((nt + 15) / 16) {
+        case 1: halves(pf_int<1>{}); break;
+#if PF_TILES > 2
+        case 2: halves(pf_int<2>{}); break;
+        case 3: halves(pf_int<3>{}); break;
+#endif
+        default: halves(pf_int<PF_TILES>{}); break;
     }
     __syncthreads();   // the staging area becomes H
-    // H = silu(gate) * up for (token 16 a + 4 kq + r, feature 16 wave + n), then per-32 quantization over features
+    if constexpr (NWV == 8) {
+        // the second half's partial sums go through LDS to the wave that holds the first half's
+        float (*pg)[65] = (float (*)[65]) (stage + PF_TOK * 65 * sizeof(float));
+        float (*pu)[65] = (float (*)[65]) (stage + 2 * PF_TOK * 65 * sizeof(float));
+        if (kh == 1) {
 #pragma unroll
-    for (int a = 0; a < PF_TILES; a++)
+            for (int a = 0; a < PF_TILES; a++)
 #pragma unroll
-        for (int r = 0; r < 4; r++) hs[16 * a + 4 * kq + r][16 * wave + n] = (accg[a][r] / (1.0f + expf(-accg[a][r]))) * accu[a][r];
+                for (int r = 0; r < 4; r++) {
+                    pg[16 * a + 4 * kq + r][16 * rw + n] = accg[a][r];
+                    pu[16 * a + 4 * kq + r][16 * rw + n] = accu[a][r];
+                }
+        }
+        __syncthreads();
+        if (kh == 0) {
+#pragma unroll
+            for (int a = 0; a < PF_TILES; a++)
+#pragma unroll
+                for (int r = 0; r < 4; r++) {
+                    accg[a][r] += pg[16 * a + 4 * kq + r][16 * rw + n];
+                    accu[a][r] += pu[16 * a + 4 * kq + r][16 * rw + n];
+                }
+        }
+    }
+    // H = silu(gate) * up for (token 16 a + 4 kq + r, feature 16 rw + n), then per-32 quantization over features
+    if (kh == 0) {
+#pragma unroll
+        for (int a = 0; a < PF_TILES; a++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) hs[16 * a + 4 * kq + r][16 * rw + n] = (accg[a][r] / (1.0f + expf(-accg[a][r]))) * accu[a][r];
+    }
     __syncthreads();
     if (tid < 2 * PF_TOK) {
         const u32 t = tid >> 1, half = tid & 1;
@@ -395,6 +458,18 @@ extern "C" __global__ void __launch_bounds__(256, 2) prefill_gate_up_iq3_s(const
             hd[(u64) p * (ff / 32) + rbx * 2 + half] = dd;
         }
     }
+}
+
+extern "C" __global__ void __launch_bounds__(512, 4) prefill_gate_up_iq3_s(const u64* eaddr, const u64* sh_addr, const u32* offs, const u32* list,
+                                                                        const u32* items, const i8* xq, const float* xd, i8* hq, float* hd, u32 ne,
+                                                                        u32 k, u32 npairs, u32 hidden, u32 ff) {
+    prefill_gate_up_iq3_s_body<8>(eaddr, sh_addr, offs, list, items, xq, xd, hq, hd, ne, k, npairs, hidden, ff);
+}
+// The same with four waves a workgroup (block 256), every wave the whole of its rows' blocks: kept for comparisons.
+extern "C" __global__ void __launch_bounds__(256, 2) prefill_gate_up_iq3_s_w4(const u64* eaddr, const u64* sh_addr, const u32* offs, const u32* list,
+                                                                           const u32* items, const i8* xq, const float* xd, i8* hq, float* hd, u32 ne,
+                                                                           u32 k, u32 npairs, u32 hidden, u32 ff) {
+    prefill_gate_up_iq3_s_body<4>(eaddr, sh_addr, offs, list, items, xq, xd, hq, hd, ne, k, npairs, hidden, ff);
 }
 
 // Work item blockIdx.y: down rows of the expert against its pairs' H: eo[pair][hidden], unweighted (cpu_expert.rs:316-339).
